@@ -1,0 +1,218 @@
+/*
+ * mi_mlp.h -- C ABI of libmi_mlp.so: the MI355X (gfx950) implementation of the tbb_test MLP
+ * training step (forward GEMM, the two backward GEMMs, gradient reduce + SGD).
+ *
+ * The reference has no FFI: its hot path is three cblas_sgemm call sites and two hand-written
+ * all-reduce functions, called from the iteration loop of mlp_omp.cc / mlp_tbb.cc.  Each entry
+ * point below names the reference call site it stands in for.
+ *
+ * Conventions
+ *   - every function returns MI_OK (0) or a negative mi_status; mi_last_error() gives the text
+ *     of the most recent failure on the calling thread.  Nothing here aborts the process.
+ *   - all matrices are row-major with an explicit leading dimension in ELEMENTS.
+ *   - "device pointer" = memory of the current HIP device (hipMalloc, mi_malloc, or a
+ *     torch tensor's data_ptr()); "host pointer" = ordinary pageable or pinned host memory.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Raw operations are
+ *     asynchronous with respect to the host.
+ *   - a handle is not thread-safe; distinct handles may be used from distinct threads.
+ */
+#ifndef MI_MLP_H
+#define MI_MLP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum mi_status {
+  MI_OK = 0,
+  MI_ERR_INVALID = -1,     /* bad argument (shape, alignment, null pointer, index out of range) */
+  MI_ERR_HIP = -2,         /* a HIP runtime call failed; mi_last_error() carries hipGetErrorString */
+  MI_ERR_NO_DEVICE = -3,   /* no gfx950 device visible */
+  MI_ERR_UNSUPPORTED = -4  /* valid request this build does not implement */
+} mi_status;
+
+typedef enum mi_dtype {
+  MI_F32 = 0, /* fp32 storage, fp32 MFMA */
+  MI_BF16 = 1 /* bf16 activations and weight shadow, fp32 MFMA accumulation, fp32 master weights,
+                 fp32 gradients and reduce */
+} mi_dtype;
+
+/* mi_mlp_create flags */
+#define MI_FLAG_RELU_LAST 0x1u   /* ReLU after the last layer too (c2_bench/mlp_caffe2.py:215-217);
+                                    default: ReLU between layers only */
+#define MI_FLAG_NO_GRAPH 0x2u    /* mi_mlp_step launches kernels one by one instead of replaying a
+                                    captured HIP graph */
+#define MI_FLAG_PER_LAYER_UPDATE 0x4u /* reduce + SGD of layer l+1 is issued right after layer
+                                    l+1's input-gradient GEMM on a second stream, so it overlaps
+                                    layer l's GEMMs -- the schedule of OVERLAP_ALL_REDUCE,
+                                    mlp_omp.cc:601-615,692-723 -- instead of one launch over all
+                                    layers at the end of the step */
+
+/* Timing slots, same names and order as the reference's enum Breakdown
+ * (mlp_bench_common.h:12-20). */
+enum {
+  MI_FWD = 0,
+  MI_WGT_GRAD,
+  MI_BWD,
+  MI_WGT_UPDATE,
+  MI_WGT_UPDATE_REDUCE_SCATTER, /* always 0 on one GPU: there is no scatter phase */
+  MI_WGT_UPDATE_ALLGATHER,      /* always 0 on one GPU: there is one copy of W    */
+  MI_NUM_BREAKDOWNS
+};
+
+/* ------------------------------------------------------------------------------------------ */
+/* library / device                                                                           */
+
+const char* mi_last_error(void);
+
+/* Name, compute-unit count, peak engine clock (MHz) and memory size of the current device. */
+int mi_device_info(char* name, int name_len, int* num_cus, int* clock_mhz, size_t* hbm_bytes);
+
+/* Thin device-memory helpers so that a host program needs no HIP headers. */
+int mi_malloc(void** dptr, size_t bytes);
+int mi_free(void* dptr);
+int mi_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int mi_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int mi_memset(void* dptr, int byte, size_t bytes);
+int mi_stream_sync(void* stream);
+
+/* Tuning hook: force tile configuration `variant` of the MFMA GEMM for kind 0 (nt), 1 (nn) or
+ * 2 (tn); 0 restores the automatic choice.  A shape the forced configuration cannot tile falls
+ * back to the any-shape kernel.  Process-wide; not meant for production callers. */
+int mi_set_gemm_variant(int kind, int variant);
+
+/* ------------------------------------------------------------------------------------------ */
+/* raw operations on device pointers: one per reference call site                             */
+
+/*
+ * Forward:  C[M x N] = A[M x K] * B[N x K]^T (+ bias[N]) , optional ReLU.
+ * Replaces cblas_sgemm(RowMajor, NoTrans, Trans, ...) at mlp_omp.cc:474-488 / mlp_tbb.cc:860-874
+ * (A = activations[l], B = weights[l], C = activations[l+1]); one call covers the whole
+ * M = R*B batch instead of one call per thread block.  bias may be NULL.
+ */
+int mi_sgemm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                int ldc, const float* bias, int relu, void* stream);
+
+/*
+ * Input gradient:  C[M x N] = A[M x K] * B[K x N], optionally multiplied element-wise by
+ * [mask_src > 0] (mask_src[M x N], leading dimension ldmask; NULL = no mask).
+ * Replaces cblas_sgemm(RowMajor, NoTrans, NoTrans, ...) at mlp_omp.cc:657-671 /
+ * mlp_tbb.cc:1144-1158 (A = dY of layer l, B = weights[l], C = dX).
+ */
+int mi_sgemm_nn(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                int ldc, const float* mask_src, int ldmask, void* stream);
+
+/*
+ * Weight gradient, one GEMM per replica in a single launch:
+ *   for r in [0, R):  C_r[M x N] = A[r*K .. (r+1)*K, 0..M)^T * B[r*K .. (r+1)*K, 0..N)
+ *                     colsum_r[M] = sum over those K rows of A          (if colsum != NULL)
+ * with C_r = C + r*strideC and colsum_r = colsum + r*stride_colsum (strides in elements).
+ * Replaces cblas_sgemm(RowMajor, Trans, NoTrans, ...) at mlp_omp.cc:565-580 /
+ * mlp_tbb.cc:1029-1043, including the split of the batch (k) over sockets at
+ * mlp_omp.cc:529-531: replica r = socket r, A = dY of layer l, B = activations[l],
+ * C_r = the socket's own slice of weight_grads[l].  colsum is the bias gradient.
+ */
+int mi_sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
+                float* C, int ldc, long long strideC, float* colsum, long long stride_colsum,
+                void* stream);
+
+/*
+ * Gradient reduce with the SGD update fused in, over a flat array of n floats:
+ *   W[i] = fma(-lr, G[i] + G[stride+i] + ... + G[(R-1)*stride+i], W[i])
+ * fp32 adds in replica order, one fused multiply-add (the arithmetic of mlp_omp.cc:140-143 and
+ * :242-250).  Replaces update_weight_reduce_scatter + update_weight_allgather
+ * (mlp_omp.cc:56-169,171-295; mlp_tbb.cc:142-456): with all R replicas' gradients resident in
+ * one HBM there is nothing to scatter or gather, and one W instead of R copies.
+ */
+int mi_reduce_sgd_raw(float* W, const float* G, size_t n, size_t replica_stride, int R, float lr,
+                      void* stream);
+
+/* Same, additionally writing the updated weights rounded to bf16 (round-to-nearest-even) into
+ * W_bf16[n] (the operand copy the bf16 GEMMs read). */
+int mi_reduce_sgd_bf16_raw(float* W, void* W_bf16, const float* G, size_t n, size_t replica_stride,
+                           int R, float lr, void* stream);
+
+/* bf16 variants of the three GEMMs: A, B (and C for nt/nn) are bf16 stored as 16-bit words,
+ * products accumulate in fp32.  mi_hgemm_tn writes fp32 gradients. */
+int mi_hgemm_nt(int M, int N, int K, const void* A, int lda, const void* B, int ldb, void* C,
+                int ldc, const float* bias, int relu, void* stream);
+int mi_hgemm_nn(int M, int N, int K, const void* A, int lda, const void* B, int ldb, void* C,
+                int ldc, const void* mask_src, int ldmask, void* stream);
+int mi_hgemm_tn(int R, int M, int N, int K, const void* A, int lda, const void* B, int ldb,
+                float* C, int ldc, long long strideC, float* colsum, long long stride_colsum,
+                void* stream);
+
+/* fp32 <-> bf16 conversion of n contiguous elements on the device. */
+int mi_convert_f32_to_bf16(void* dst_bf16, const float* src, size_t n, void* stream);
+int mi_convert_bf16_to_f32(float* dst, const void* src_bf16, size_t n, void* stream);
+
+/* ------------------------------------------------------------------------------------------ */
+/* handle API: the whole model resident in HBM                                                */
+
+typedef struct mi_mlp mi_mlp;
+
+/*
+ * Allocates the model on the current device: L fully-connected layers of widths
+ * nfeatures[0..L] (layer l maps nfeatures[l] -> nfeatures[l+1], weight W_l is
+ * [nfeatures[l+1] x nfeatures[l]] as at mlp_omp.cc:395-396), R data-parallel replicas of
+ * batch_per_replica rows each (replica r owns rows [r*B, (r+1)*B) of every activation, the
+ * split of Partition.cc:25-27).  Device state: one parameter arena (all W_l and b_l), R gradient
+ * arenas of the same layout, L+1 activation buffers and two gradient ping-pong buffers.
+ * Stands in for the allocation block of main(), mlp_omp.cc:390-409.
+ */
+int mi_mlp_create(mi_mlp** h, int L, const int* nfeatures, int batch_per_replica, int R, int dtype,
+                  unsigned flags);
+int mi_mlp_destroy(mi_mlp* h);
+
+/* Host -> device uploads.  ld in elements; b may be NULL (bias = 0).  Stand in for
+ * init_matrices(), mlp_bench_common.cc:16-33. */
+int mi_mlp_set_weights(mi_mlp* h, int l, const float* W, int ld, const float* b);
+int mi_mlp_set_input(mi_mlp* h, const float* X, int ld);
+int mi_mlp_set_dy(mi_mlp* h, const float* dY, int ld);
+
+/* Per-operation entry points, asynchronous on the handle's stream.  Backward runs from the
+ * last layer down; mi_fc_dgrad(l) consumes the gradient produced by mi_fc_dgrad(l+1) (or the
+ * uploaded dY for l = L-1). */
+int mi_fc_forward(mi_mlp* h, int l); /* mlp_omp.cc:441-510 */
+int mi_fc_wgrad(mi_mlp* h, int l);   /* mlp_omp.cc:513-600, all R replicas; also the bias gradient */
+int mi_fc_bgrad(mi_mlp* h, int l);   /* bias gradient alone (column sums of the layer's dZ) */
+int mi_fc_dgrad(mi_mlp* h, int l);   /* mlp_omp.cc:619-691 */
+int mi_reduce_sgd(mi_mlp* h, float lr);                /* all layers, one launch */
+int mi_reduce_sgd_layer(mi_mlp* h, int l, float lr);   /* one layer (W_l and b_l) */
+
+/* One full step: forward over all layers, backward over all layers, reduce + SGD
+ * (the body of the iteration loop, mlp_omp.cc:435-737). Asynchronous; mi_mlp_sync waits. */
+int mi_mlp_step(mi_mlp* h, float lr);
+int mi_mlp_sync(mi_mlp* h);
+
+/* Device -> host downloads (synchronous).  Activations and gradients come back as fp32 whatever
+ * the handle's dtype.  l in [0, L] for activations (0 = input), r in [0, R). */
+int mi_mlp_get_activation(mi_mlp* h, int l, float* dst, int ld);
+int mi_mlp_get_weight(mi_mlp* h, int l, float* dst, int ld);
+int mi_mlp_get_bias(mi_mlp* h, int l, float* dst);
+int mi_mlp_get_wgrad(mi_mlp* h, int l, int r, float* dst, int ld);
+int mi_mlp_get_bgrad(mi_mlp* h, int l, int r, float* dst);
+int mi_mlp_get_dx(mi_mlp* h, float* dst, int ld);
+
+/* Number of parameters P = sum_l (N_l*N_{l+1} + N_{l+1}) and the padded element stride between
+ * consecutive replicas' gradient arenas. */
+int mi_mlp_param_count(mi_mlp* h, size_t* params, size_t* replica_stride);
+
+/*
+ * Per-phase device timing with HIP events on the handle's stream (the role of sum_times /
+ * dsecnd() in mlp_omp.cc:490-508,582-600,673-691,161-168).  While enabled, every kernel of
+ * mi_mlp_step and of the per-operation entry points is bracketed by an event pair.
+ * mi_mlp_get_timings synchronises and writes accumulated milliseconds as
+ * ms[breakdown * L + layer]; the single all-layer reduce launch is booked under
+ * MI_WGT_UPDATE, layer 0.  launches[] (same indexing, may be NULL) receives launch counts.
+ */
+int mi_mlp_enable_timing(mi_mlp* h, int on);
+int mi_mlp_reset_timings(mi_mlp* h);
+int mi_mlp_get_timings(mi_mlp* h, double* ms, long long* launches);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_MLP_H */

@@ -1,0 +1,732 @@
+// Implementation of the C ABI declared in include/mi_mlp.h: argument checking, device state of
+// one model (parameter arena, R gradient arenas, activations), the step schedule, event timing
+// and HIP-graph replay.  The arithmetic lives in gemm_f32.hip, gemm_bf16.hip and reduce_sgd.hip.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "kernels.h"
+#include "mi_mlp.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(MI_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define MI_HIP(call)                                  \
+  do {                                                \
+    hipError_t e_ = (call);                           \
+    if (e_ != hipSuccess) return hip_fail(e_, #call); \
+  } while (0)
+
+#define MI_REQUIRE(cond, ...) \
+  do {                        \
+    if (!(cond)) return fail(MI_ERR_INVALID, __VA_ARGS__); \
+  } while (0)
+
+int g_variant[3] = {0, 0, 0};  // forced tile configuration per GEMM kind (nt, nn, tn); 0 = automatic
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------------
+// model state
+
+struct mi_mlp {
+  int L = 0, B = 0, R = 0, dtype = MI_F32;
+  unsigned flags = 0;
+  int MB = 0;  // rows of every activation = R * B
+  std::vector<int> nf;
+  size_t P = 0;        // parameter count, padding excluded
+  size_t stride = 0;   // floats per arena (segments padded to 256 bytes)
+  std::vector<size_t> woff, boff;  // float offsets of W_l / b_l inside an arena
+  float* params = nullptr;    // [stride]
+  float* grads = nullptr;     // [R * stride]
+  uint16_t* params16 = nullptr;  // bf16 copy of params (dtype bf16)
+  std::vector<void*> acts;    // L+1 buffers [MB x nf[l]], fp32 or bf16
+  void* dy = nullptr;         // upstream gradient [MB x nf[L]]
+  void* dz[2] = {nullptr, nullptr};  // gradient ping-pong [MB x max width]
+  void* dx = nullptr;         // gradient w.r.t. the input [MB x nf[0]]
+  float* staging = nullptr;   // fp32 bounce buffer for bf16 uploads/downloads [MB x max width] or one W
+  size_t staging_elems = 0;
+  hipStream_t stream = nullptr, stream2 = nullptr;
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  std::vector<hipEvent_t> ev_layer;  // per-layer "input-gradient GEMM done" (overlapped update)
+
+  // timing
+  bool timing = false;
+  struct Pair { hipEvent_t a, b; int slot; };
+  std::vector<Pair> pending;
+  std::vector<hipEvent_t> free_events;
+  std::vector<double> ms;
+  std::vector<long long> launches;
+
+  // graph replay
+  hipGraphExec_t graph_exec = nullptr;
+  float graph_lr = 0.0f;
+  int eager_steps = 0;
+
+  size_t esize() const { return dtype == MI_BF16 ? 2 : 4; }
+  size_t maxw() const {
+    size_t m = 0;
+    for (int v : nf) m = v > (int)m ? (size_t)v : m;
+    return m;
+  }
+};
+
+namespace {
+
+int check_handle(mi_mlp* h) {
+  if (!h) return fail(MI_ERR_INVALID, "null handle");
+  return MI_OK;
+}
+int check_layer(mi_mlp* h, int l, int hi_inclusive) {
+  if (!h) return fail(MI_ERR_INVALID, "null handle");
+  if (l < 0 || l > hi_inclusive) return fail(MI_ERR_INVALID, "layer index %d out of range [0,%d]", l, hi_inclusive);
+  return MI_OK;
+}
+
+// event timing ------------------------------------------------------------------------------------
+int harvest(mi_mlp* h) {
+  if (h->pending.empty()) return MI_OK;
+  MI_HIP(hipStreamSynchronize(h->stream));
+  if (h->stream2) MI_HIP(hipStreamSynchronize(h->stream2));
+  for (auto& p : h->pending) {
+    float t = 0.0f;
+    MI_HIP(hipEventElapsedTime(&t, p.a, p.b));
+    h->ms[p.slot] += (double)t;
+    h->launches[p.slot] += 1;
+    h->free_events.push_back(p.a);
+    h->free_events.push_back(p.b);
+  }
+  h->pending.clear();
+  return MI_OK;
+}
+
+int get_event(mi_mlp* h, hipEvent_t* ev) {
+  if (h->free_events.empty()) {
+    MI_HIP(hipEventCreate(ev));
+  } else {
+    *ev = h->free_events.back();
+    h->free_events.pop_back();
+  }
+  return MI_OK;
+}
+
+struct TimedScope {
+  mi_mlp* h;
+  hipStream_t s;
+  hipEvent_t a = nullptr, b = nullptr;
+  int slot;
+  int status = MI_OK;
+  TimedScope(mi_mlp* h_, hipStream_t s_, int breakdown, int layer) : h(h_), s(s_), slot(breakdown * h_->L + layer) {
+    if (!h->timing) return;
+    if (h->pending.size() >= 8192) status = harvest(h);
+    if (status == MI_OK) status = get_event(h, &a);
+    if (status == MI_OK) status = get_event(h, &b);
+    if (status == MI_OK && hipEventRecord(a, s) != hipSuccess) status = fail(MI_ERR_HIP, "hipEventRecord failed");
+  }
+  int finish() {
+    if (!h->timing || status != MI_OK) return status;
+    if (hipEventRecord(b, s) != hipSuccess) return fail(MI_ERR_HIP, "hipEventRecord failed");
+    h->pending.push_back({a, b, slot});
+    return MI_OK;
+  }
+};
+
+// operations on the handle ----------------------------------------------------------------------
+const void* dz_of_layer(mi_mlp* h, int l) {
+  // gradient w.r.t. the pre-activation output of layer l
+  if (l == h->L - 1 && !(h->flags & MI_FLAG_RELU_LAST)) return h->dy;
+  return h->dz[l & 1];
+}
+
+int op_forward(mi_mlp* h, int l, hipStream_t s) {
+  const int relu = (l < h->L - 1) || (h->flags & MI_FLAG_RELU_LAST);
+  TimedScope ts(h, s, MI_FWD, l);
+  if (ts.status) return ts.status;
+  hipError_t e;
+  if (h->dtype == MI_F32) {
+    e = mi::sgemm_nt(h->MB, h->nf[l + 1], h->nf[l], (const float*)h->acts[l], h->nf[l], h->params + h->woff[l],
+                     h->nf[l], (float*)h->acts[l + 1], h->nf[l + 1], h->params + h->boff[l], relu, s, g_variant[0]);
+  } else {
+    return fail(MI_ERR_UNSUPPORTED, "bf16 forward is not implemented in this build");
+  }
+  if (e != hipSuccess) return hip_fail(e, "forward GEMM launch");
+  return ts.finish();
+}
+
+int op_wgrad(mi_mlp* h, int l, hipStream_t s, bool with_bias) {
+  const float* g0 = h->grads + h->woff[l];
+  TimedScope ts(h, s, MI_WGT_GRAD, l);
+  if (ts.status) return ts.status;
+  hipError_t e;
+  if (h->dtype == MI_F32) {
+    e = mi::sgemm_tn(h->R, h->nf[l + 1], h->nf[l], h->B, (const float*)dz_of_layer(h, l), h->nf[l + 1],
+                     (const float*)h->acts[l], h->nf[l], const_cast<float*>(g0), h->nf[l], (long long)h->stride, s,
+                     g_variant[2]);
+    if (e == hipSuccess && with_bias)
+      e = mi::colsum_f32(h->R, h->nf[l + 1], h->B, (const float*)dz_of_layer(h, l), h->nf[l + 1],
+                         h->grads + h->boff[l], (long long)h->stride, s);
+  } else {
+    return fail(MI_ERR_UNSUPPORTED, "bf16 weight gradient is not implemented in this build");
+  }
+  if (e != hipSuccess) return hip_fail(e, "weight-gradient GEMM launch");
+  return ts.finish();
+}
+
+int op_bgrad(mi_mlp* h, int l, hipStream_t s) {
+  if (h->dtype != MI_F32) return fail(MI_ERR_UNSUPPORTED, "bf16 bias gradient is not implemented in this build");
+  hipError_t e = mi::colsum_f32(h->R, h->nf[l + 1], h->B, (const float*)dz_of_layer(h, l), h->nf[l + 1],
+                                h->grads + h->boff[l], (long long)h->stride, s);
+  if (e != hipSuccess) return hip_fail(e, "bias-gradient launch");
+  return MI_OK;
+}
+
+int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
+  TimedScope ts(h, s, MI_BWD, l);
+  if (ts.status) return ts.status;
+  void* out = (l == 0) ? h->dx : h->dz[(l - 1) & 1];
+  const void* mask = (l == 0) ? nullptr : h->acts[l];
+  hipError_t e;
+  if (h->dtype == MI_F32) {
+    e = mi::sgemm_nn(h->MB, h->nf[l], h->nf[l + 1], (const float*)dz_of_layer(h, l), h->nf[l + 1],
+                     h->params + h->woff[l], h->nf[l], (float*)out, h->nf[l], (const float*)mask, h->nf[l], s,
+                     g_variant[1]);
+  } else {
+    return fail(MI_ERR_UNSUPPORTED, "bf16 input gradient is not implemented in this build");
+  }
+  if (e != hipSuccess) return hip_fail(e, "input-gradient GEMM launch");
+  return ts.finish();
+}
+
+int op_update(mi_mlp* h, int l_or_all, float lr, hipStream_t s) {
+  size_t off = 0, n = h->stride;
+  int layer_slot = 0;
+  if (l_or_all >= 0) {
+    off = h->woff[l_or_all];
+    n = (l_or_all + 1 < h->L ? h->woff[l_or_all + 1] : h->stride) - off;
+    layer_slot = l_or_all;
+  }
+  TimedScope ts(h, s, MI_WGT_UPDATE, layer_slot);
+  if (ts.status) return ts.status;
+  hipError_t e = mi::reduce_sgd(h->params + off, h->params16 ? h->params16 + off : nullptr, h->grads + off, n,
+                                h->stride, h->R, lr, s);
+  if (e != hipSuccess) return hip_fail(e, "reduce+SGD launch");
+  return ts.finish();
+}
+
+// dZ of the last layer when it carries a ReLU: dY masked by the sign of the output
+__global__ __launch_bounds__(256) void mask_copy_kernel(float* __restrict__ dst, const float* __restrict__ g,
+                                                        const float* __restrict__ act, size_t n) {
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step)
+    dst[i] = act[i] > 0.0f ? g[i] : 0.0f;
+}
+
+int op_last_mask(mi_mlp* h, hipStream_t s) {
+  if (!(h->flags & MI_FLAG_RELU_LAST)) return MI_OK;
+  if (h->dtype != MI_F32) return fail(MI_ERR_UNSUPPORTED, "bf16 ReLU-last is not implemented in this build");
+  const size_t n = (size_t)h->MB * h->nf[h->L];
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(mask_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float*)h->dz[(h->L - 1) & 1],
+                     (const float*)h->dy, (const float*)h->acts[h->L], n);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e, "mask launch");
+  return MI_OK;
+}
+
+// Enqueues one whole step.  With MI_FLAG_PER_LAYER_UPDATE the update of layer l runs on the second
+// stream as soon as layer l's input-gradient GEMM (the last reader of W_l) has finished, and the
+// main stream waits for all updates at the end.
+int enqueue_step(mi_mlp* h, float lr) {
+  hipStream_t s = h->stream;
+  int rc;
+  for (int l = 0; l < h->L; ++l)
+    if ((rc = op_forward(h, l, s))) return rc;
+  if ((rc = op_last_mask(h, s))) return rc;
+  const bool overlap = (h->flags & MI_FLAG_PER_LAYER_UPDATE) != 0;
+  for (int l = h->L - 1; l >= 0; --l) {
+    if ((rc = op_wgrad(h, l, s, true))) return rc;
+    if ((rc = op_dgrad(h, l, s))) return rc;
+    if (overlap) {
+      MI_HIP(hipEventRecord(h->ev_layer[l], s));
+      MI_HIP(hipStreamWaitEvent(h->stream2, h->ev_layer[l], 0));
+      if ((rc = op_update(h, l, lr, h->stream2))) return rc;
+    }
+  }
+  if (overlap) {
+    MI_HIP(hipEventRecord(h->ev_join, h->stream2));
+    MI_HIP(hipStreamWaitEvent(s, h->ev_join, 0));
+  } else {
+    if ((rc = op_update(h, -1, lr, s))) return rc;
+  }
+  return MI_OK;
+}
+
+void drop_graph(mi_mlp* h) {
+  if (h->graph_exec) {
+    (void)hipGraphExecDestroy(h->graph_exec);
+    h->graph_exec = nullptr;
+  }
+}
+
+// host <-> device copies of one [rows x cols] matrix with arbitrary host leading dimension
+int upload_matrix(mi_mlp* h, void* dst, const float* src, int rows, int cols, int ld, bool as_bf16) {
+  MI_REQUIRE(src != nullptr, "null host pointer");
+  MI_REQUIRE(ld >= cols, "leading dimension %d smaller than %d columns", ld, cols);
+  if (!as_bf16) {
+    MI_HIP(hipMemcpy2DAsync(dst, (size_t)cols * 4, src, (size_t)ld * 4, (size_t)cols * 4, rows,
+                            hipMemcpyHostToDevice, h->stream));
+    MI_HIP(hipStreamSynchronize(h->stream));
+    return MI_OK;
+  }
+  MI_REQUIRE((size_t)rows * cols <= h->staging_elems, "staging buffer too small");
+  MI_HIP(hipMemcpy2DAsync(h->staging, (size_t)cols * 4, src, (size_t)ld * 4, (size_t)cols * 4, rows,
+                          hipMemcpyHostToDevice, h->stream));
+  hipError_t e = mi::convert_f32_to_bf16((uint16_t*)dst, h->staging, (size_t)rows * cols, h->stream);
+  if (e != hipSuccess) return hip_fail(e, "convert launch");
+  MI_HIP(hipStreamSynchronize(h->stream));
+  return MI_OK;
+}
+
+int download_matrix(mi_mlp* h, float* dst, const void* src, int rows, int cols, int ld, bool from_bf16) {
+  MI_REQUIRE(dst != nullptr, "null host pointer");
+  MI_REQUIRE(ld >= cols, "leading dimension %d smaller than %d columns", ld, cols);
+  MI_HIP(hipStreamSynchronize(h->stream));
+  if (h->stream2) MI_HIP(hipStreamSynchronize(h->stream2));
+  const void* from = src;
+  if (from_bf16) {
+    MI_REQUIRE((size_t)rows * cols <= h->staging_elems, "staging buffer too small");
+    hipError_t e = mi::convert_bf16_to_f32(h->staging, (const uint16_t*)src, (size_t)rows * cols, h->stream);
+    if (e != hipSuccess) return hip_fail(e, "convert launch");
+    from = h->staging;
+  }
+  MI_HIP(hipMemcpy2DAsync(dst, (size_t)ld * 4, from, (size_t)cols * 4, (size_t)cols * 4, rows,
+                          hipMemcpyDeviceToHost, h->stream));
+  MI_HIP(hipStreamSynchronize(h->stream));
+  return MI_OK;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------------
+extern "C" {
+
+const char* mi_last_error(void) { return g_last_error.c_str(); }
+
+int mi_device_info(char* name, int name_len, int* num_cus, int* clock_mhz, size_t* hbm_bytes) {
+  int dev = 0, count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count == 0) return fail(MI_ERR_NO_DEVICE, "no HIP device visible");
+  MI_HIP(hipGetDevice(&dev));
+  hipDeviceProp_t prop;
+  MI_HIP(hipGetDeviceProperties(&prop, dev));
+  if (name && name_len > 0) snprintf(name, (size_t)name_len, "%s (%s)", prop.name, prop.gcnArchName);
+  if (num_cus) *num_cus = prop.multiProcessorCount;
+  if (clock_mhz) *clock_mhz = prop.clockRate / 1000;
+  if (hbm_bytes) *hbm_bytes = prop.totalGlobalMem;
+  return MI_OK;
+}
+
+int mi_malloc(void** dptr, size_t bytes) {
+  MI_REQUIRE(dptr != nullptr, "null output pointer");
+  *dptr = nullptr;
+  if (bytes == 0) return MI_OK;
+  MI_HIP(hipMalloc(dptr, bytes));
+  return MI_OK;
+}
+int mi_free(void* dptr) {
+  if (dptr) MI_HIP(hipFree(dptr));
+  return MI_OK;
+}
+int mi_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+  if (bytes) MI_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+  return MI_OK;
+}
+int mi_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+  if (bytes) MI_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+  return MI_OK;
+}
+int mi_memset(void* dptr, int byte, size_t bytes) {
+  if (bytes) MI_HIP(hipMemset(dptr, byte, bytes));
+  return MI_OK;
+}
+int mi_stream_sync(void* stream) {
+  MI_HIP(hipStreamSynchronize(as_stream(stream)));
+  return MI_OK;
+}
+
+int mi_set_gemm_variant(int kind, int variant) {
+  MI_REQUIRE(kind >= 0 && kind < 3, "kind must be 0 (nt), 1 (nn) or 2 (tn)");
+  g_variant[kind] = variant;
+  return MI_OK;
+}
+
+// ---- raw operations -----------------------------------------------------------------------------
+
+static int check_gemm(int M, int N, int K, const void* A, int lda, int min_lda, const void* B, int ldb, int min_ldb,
+                      const void* C, int ldc) {
+  MI_REQUIRE(M >= 0 && N >= 0 && K >= 0, "negative dimension (M=%d N=%d K=%d)", M, N, K);
+  if (M == 0 || N == 0) return MI_OK;
+  MI_REQUIRE(C != nullptr, "null C");
+  MI_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "null operand");
+  MI_REQUIRE(lda >= min_lda, "lda %d < %d", lda, min_lda);
+  MI_REQUIRE(ldb >= min_ldb, "ldb %d < %d", ldb, min_ldb);
+  MI_REQUIRE(ldc >= N, "ldc %d < N %d", ldc, N);
+  return MI_OK;
+}
+
+int mi_sgemm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                const float* bias, int relu, void* stream) {
+  if (int rc = check_gemm(M, N, K, A, lda, K, B, ldb, K, C, ldc)) return rc;
+  hipError_t e = mi::sgemm_nt(M, N, K, A, lda, B, ldb, C, ldc, bias, relu, as_stream(stream), g_variant[0]);
+  if (e != hipSuccess) return hip_fail(e, "mi_sgemm_nt launch");
+  return MI_OK;
+}
+
+int mi_sgemm_nn(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                const float* mask_src, int ldmask, void* stream) {
+  if (int rc = check_gemm(M, N, K, A, lda, K, B, ldb, N, C, ldc)) return rc;
+  MI_REQUIRE(!mask_src || ldmask >= N, "ldmask %d < N %d", ldmask, N);
+  hipError_t e = mi::sgemm_nn(M, N, K, A, lda, B, ldb, C, ldc, mask_src, ldmask, as_stream(stream), g_variant[1]);
+  if (e != hipSuccess) return hip_fail(e, "mi_sgemm_nn launch");
+  return MI_OK;
+}
+
+int mi_sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                long long strideC, float* colsum, long long stride_colsum, void* stream) {
+  MI_REQUIRE(R >= 0, "negative replica count");
+  if (R == 0) return MI_OK;
+  if (int rc = check_gemm(M, N, K, A, lda, M, B, ldb, N, C, ldc)) return rc;
+  MI_REQUIRE(R == 1 || strideC >= (long long)(M > 0 ? (size_t)(M - 1) * ldc + N : 0), "strideC overlaps replicas");
+  MI_REQUIRE(!colsum || R == 1 || stride_colsum >= M, "stride_colsum overlaps replicas");
+  hipError_t e = mi::sgemm_tn(R, M, N, K, A, lda, B, ldb, C, ldc, strideC, as_stream(stream), g_variant[2]);
+  if (e == hipSuccess && colsum) e = mi::colsum_f32(R, M, K, A, lda, colsum, stride_colsum, as_stream(stream));
+  if (e != hipSuccess) return hip_fail(e, "mi_sgemm_tn launch");
+  return MI_OK;
+}
+
+int mi_reduce_sgd_raw(float* W, const float* G, size_t n, size_t replica_stride, int R, float lr, void* stream) {
+  MI_REQUIRE(R >= 1, "R must be at least 1 (got %d)", R);
+  if (n == 0) return MI_OK;
+  MI_REQUIRE(W && G, "null pointer");
+  MI_REQUIRE(R == 1 || replica_stride >= n, "replica_stride %zu < n %zu", replica_stride, n);
+  hipError_t e = mi::reduce_sgd(W, nullptr, G, n, replica_stride, R, lr, as_stream(stream));
+  if (e != hipSuccess) return hip_fail(e, "mi_reduce_sgd_raw launch");
+  return MI_OK;
+}
+
+int mi_reduce_sgd_bf16_raw(float* W, void* W_bf16, const float* G, size_t n, size_t replica_stride, int R, float lr,
+                           void* stream) {
+  MI_REQUIRE(R >= 1, "R must be at least 1 (got %d)", R);
+  if (n == 0) return MI_OK;
+  MI_REQUIRE(W && G && W_bf16, "null pointer");
+  MI_REQUIRE(R == 1 || replica_stride >= n, "replica_stride %zu < n %zu", replica_stride, n);
+  hipError_t e = mi::reduce_sgd(W, (uint16_t*)W_bf16, G, n, replica_stride, R, lr, as_stream(stream));
+  if (e != hipSuccess) return hip_fail(e, "mi_reduce_sgd_bf16_raw launch");
+  return MI_OK;
+}
+
+int mi_hgemm_nt(int, int, int, const void*, int, const void*, int, void*, int, const float*, int, void*) {
+  return fail(MI_ERR_UNSUPPORTED, "bf16 GEMMs are not implemented in this build");
+}
+int mi_hgemm_nn(int, int, int, const void*, int, const void*, int, void*, int, const void*, int, void*) {
+  return fail(MI_ERR_UNSUPPORTED, "bf16 GEMMs are not implemented in this build");
+}
+int mi_hgemm_tn(int, int, int, int, const void*, int, const void*, int, float*, int, long long, float*, long long,
+                void*) {
+  return fail(MI_ERR_UNSUPPORTED, "bf16 GEMMs are not implemented in this build");
+}
+
+int mi_convert_f32_to_bf16(void* dst, const float* src, size_t n, void* stream) {
+  MI_REQUIRE(n == 0 || (dst && src), "null pointer");
+  hipError_t e = mi::convert_f32_to_bf16((uint16_t*)dst, src, n, as_stream(stream));
+  if (e != hipSuccess) return hip_fail(e, "convert launch");
+  return MI_OK;
+}
+int mi_convert_bf16_to_f32(float* dst, const void* src, size_t n, void* stream) {
+  MI_REQUIRE(n == 0 || (dst && src), "null pointer");
+  hipError_t e = mi::convert_bf16_to_f32(dst, (const uint16_t*)src, n, as_stream(stream));
+  if (e != hipSuccess) return hip_fail(e, "convert launch");
+  return MI_OK;
+}
+
+// ---- handle -------------------------------------------------------------------------------------
+
+int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_replica, int R, int dtype,
+                  unsigned flags) {
+  MI_REQUIRE(out != nullptr, "null output handle");
+  *out = nullptr;
+  MI_REQUIRE(L >= 1 && L <= 4096, "layer count %d out of range", L);
+  MI_REQUIRE(nfeatures != nullptr, "null nfeatures");
+  MI_REQUIRE(batch_per_replica >= 1 && R >= 1, "batch_per_replica and R must be positive");
+  MI_REQUIRE((long long)batch_per_replica * R <= 0x7fffffffLL, "R * batch overflows int");
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "unknown dtype %d", dtype);
+  for (int l = 0; l <= L; ++l) MI_REQUIRE(nfeatures[l] >= 1, "nfeatures[%d] = %d must be positive", l, nfeatures[l]);
+  if (dtype == MI_BF16) return fail(MI_ERR_UNSUPPORTED, "the bf16 model is not implemented in this build");
+
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count == 0) return fail(MI_ERR_NO_DEVICE, "no HIP device visible");
+
+  mi_mlp* h = new (std::nothrow) mi_mlp;
+  MI_REQUIRE(h != nullptr, "out of host memory");
+  h->L = L;
+  h->B = batch_per_replica;
+  h->R = R;
+  h->MB = batch_per_replica * R;
+  h->dtype = dtype;
+  h->flags = flags;
+  h->nf.assign(nfeatures, nfeatures + L + 1);
+  h->woff.resize(L);
+  h->boff.resize(L);
+  size_t off = 0;
+  for (int l = 0; l < L; ++l) {
+    h->woff[l] = off;
+    off = round_up(off + (size_t)h->nf[l + 1] * h->nf[l], 64);
+    h->boff[l] = off;
+    off = round_up(off + (size_t)h->nf[l + 1], 64);
+    h->P += (size_t)h->nf[l + 1] * h->nf[l] + h->nf[l + 1];
+  }
+  h->stride = off;
+  h->ms.assign((size_t)MI_NUM_BREAKDOWNS * L, 0.0);
+  h->launches.assign((size_t)MI_NUM_BREAKDOWNS * L, 0);
+
+  int rc = MI_OK;
+  auto alloc = [&](void** p, size_t bytes) {
+    if (rc != MI_OK) return;
+    hipError_t e = hipMalloc(p, bytes);
+    if (e != hipSuccess) { rc = hip_fail(e, "hipMalloc"); return; }
+    e = hipMemset(*p, 0, bytes);
+    if (e != hipSuccess) rc = hip_fail(e, "hipMemset");
+  };
+  const size_t es = h->esize();
+  alloc((void**)&h->params, h->stride * 4);
+  alloc((void**)&h->grads, h->stride * 4 * (size_t)R);
+  h->acts.assign(L + 1, nullptr);
+  for (int l = 0; l <= L; ++l) alloc(&h->acts[l], (size_t)h->MB * h->nf[l] * es);
+  alloc(&h->dy, (size_t)h->MB * h->nf[L] * es);
+  alloc(&h->dz[0], (size_t)h->MB * h->maxw() * es);
+  alloc(&h->dz[1], (size_t)h->MB * h->maxw() * es);
+  alloc(&h->dx, (size_t)h->MB * h->nf[0] * es);
+  if (rc == MI_OK && hipDeviceSynchronize() != hipSuccess) rc = fail(MI_ERR_HIP, "hipDeviceSynchronize failed");
+  if (rc == MI_OK && hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking) != hipSuccess)
+    rc = fail(MI_ERR_HIP, "hipStreamCreate failed");
+  if (rc == MI_OK && (flags & MI_FLAG_PER_LAYER_UPDATE)) {
+    if (hipStreamCreateWithFlags(&h->stream2, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&h->ev_join, hipEventDisableTiming) != hipSuccess)
+      rc = fail(MI_ERR_HIP, "second stream setup failed");
+    h->ev_layer.assign(L, nullptr);
+    for (int l = 0; l < L && rc == MI_OK; ++l)
+      if (hipEventCreateWithFlags(&h->ev_layer[l], hipEventDisableTiming) != hipSuccess)
+        rc = fail(MI_ERR_HIP, "hipEventCreate failed");
+  }
+  if (rc != MI_OK) {
+    std::string keep = g_last_error;
+    mi_mlp_destroy(h);
+    g_last_error = keep;
+    return rc;
+  }
+  *out = h;
+  return MI_OK;
+}
+
+int mi_mlp_destroy(mi_mlp* h) {
+  if (!h) return MI_OK;
+  if (h->stream) (void)hipStreamSynchronize(h->stream);
+  if (h->stream2) (void)hipStreamSynchronize(h->stream2);
+  drop_graph(h);
+  for (auto& p : h->pending) {
+    (void)hipEventDestroy(p.a);
+    (void)hipEventDestroy(p.b);
+  }
+  for (auto e : h->free_events) (void)hipEventDestroy(e);
+  for (auto e : h->ev_layer)
+    if (e) (void)hipEventDestroy(e);
+  if (h->ev_join) (void)hipEventDestroy(h->ev_join);
+  if (h->ev_fork) (void)hipEventDestroy(h->ev_fork);
+  (void)hipFree(h->params);
+  (void)hipFree(h->grads);
+  (void)hipFree(h->params16);
+  for (void* a : h->acts) (void)hipFree(a);
+  (void)hipFree(h->dy);
+  (void)hipFree(h->dz[0]);
+  (void)hipFree(h->dz[1]);
+  (void)hipFree(h->dx);
+  (void)hipFree(h->staging);
+  if (h->stream) (void)hipStreamDestroy(h->stream);
+  if (h->stream2) (void)hipStreamDestroy(h->stream2);
+  delete h;
+  return MI_OK;
+}
+
+int mi_mlp_set_weights(mi_mlp* h, int l, const float* W, int ld, const float* b) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  if (int rc = upload_matrix(h, h->params + h->woff[l], W, h->nf[l + 1], h->nf[l], ld, false)) return rc;
+  if (b) {
+    MI_HIP(hipMemcpy(h->params + h->boff[l], b, (size_t)h->nf[l + 1] * 4, hipMemcpyHostToDevice));
+  } else {
+    MI_HIP(hipMemsetAsync(h->params + h->boff[l], 0, (size_t)h->nf[l + 1] * 4, h->stream));
+    MI_HIP(hipStreamSynchronize(h->stream));
+  }
+  return MI_OK;
+}
+
+int mi_mlp_set_input(mi_mlp* h, const float* X, int ld) {
+  if (int rc = check_handle(h)) return rc;
+  return upload_matrix(h, h->acts[0], X, h->MB, h->nf[0], ld, h->dtype == MI_BF16);
+}
+
+int mi_mlp_set_dy(mi_mlp* h, const float* dY, int ld) {
+  if (int rc = check_handle(h)) return rc;
+  return upload_matrix(h, h->dy, dY, h->MB, h->nf[h->L], ld, h->dtype == MI_BF16);
+}
+
+int mi_fc_forward(mi_mlp* h, int l) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  return op_forward(h, l, h->stream);
+}
+int mi_fc_wgrad(mi_mlp* h, int l) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  if (l == h->L - 1)
+    if (int rc = op_last_mask(h, h->stream)) return rc;
+  return op_wgrad(h, l, h->stream, true);
+}
+int mi_fc_bgrad(mi_mlp* h, int l) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  if (l == h->L - 1)
+    if (int rc = op_last_mask(h, h->stream)) return rc;
+  return op_bgrad(h, l, h->stream);
+}
+int mi_fc_dgrad(mi_mlp* h, int l) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  if (l == h->L - 1)
+    if (int rc = op_last_mask(h, h->stream)) return rc;
+  return op_dgrad(h, l, h->stream);
+}
+int mi_reduce_sgd(mi_mlp* h, float lr) {
+  if (int rc = check_handle(h)) return rc;
+  return op_update(h, -1, lr, h->stream);
+}
+int mi_reduce_sgd_layer(mi_mlp* h, int l, float lr) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  return op_update(h, l, lr, h->stream);
+}
+
+int mi_mlp_step(mi_mlp* h, float lr) {
+  if (int rc = check_handle(h)) return rc;
+  const bool use_graph = !(h->flags & MI_FLAG_NO_GRAPH) && !h->timing;
+  if (!use_graph || h->eager_steps < 1) {
+    // the first step always runs eagerly: it performs the one-time kernel attribute setup,
+    // which must not happen inside a stream capture
+    h->eager_steps++;
+    return enqueue_step(h, lr);
+  }
+  if (h->graph_exec && h->graph_lr != lr) drop_graph(h);
+  if (!h->graph_exec) {
+    hipGraph_t graph = nullptr;
+    MI_HIP(hipStreamBeginCapture(h->stream, hipStreamCaptureModeThreadLocal));
+    int rc = enqueue_step(h, lr);
+    hipError_t e = hipStreamEndCapture(h->stream, &graph);
+    if (rc != MI_OK) {
+      if (graph) (void)hipGraphDestroy(graph);
+      return rc;
+    }
+    if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture");
+    e = hipGraphInstantiate(&h->graph_exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) {
+      h->graph_exec = nullptr;
+      return hip_fail(e, "hipGraphInstantiate");
+    }
+    h->graph_lr = lr;
+  }
+  MI_HIP(hipGraphLaunch(h->graph_exec, h->stream));
+  return MI_OK;
+}
+
+int mi_mlp_sync(mi_mlp* h) {
+  if (int rc = check_handle(h)) return rc;
+  MI_HIP(hipStreamSynchronize(h->stream));
+  if (h->stream2) MI_HIP(hipStreamSynchronize(h->stream2));
+  return MI_OK;
+}
+
+int mi_mlp_get_activation(mi_mlp* h, int l, float* dst, int ld) {
+  if (int rc = check_layer(h, l, h ? h->L : 0)) return rc;
+  return download_matrix(h, dst, h->acts[l], h->MB, h->nf[l], ld, h->dtype == MI_BF16);
+}
+int mi_mlp_get_weight(mi_mlp* h, int l, float* dst, int ld) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  return download_matrix(h, dst, h->params + h->woff[l], h->nf[l + 1], h->nf[l], ld, false);
+}
+int mi_mlp_get_bias(mi_mlp* h, int l, float* dst) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  return download_matrix(h, dst, h->params + h->boff[l], 1, h->nf[l + 1], h->nf[l + 1], false);
+}
+int mi_mlp_get_wgrad(mi_mlp* h, int l, int r, float* dst, int ld) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  MI_REQUIRE(r >= 0 && r < h->R, "replica index %d out of range [0,%d)", r, h->R);
+  return download_matrix(h, dst, h->grads + (size_t)r * h->stride + h->woff[l], h->nf[l + 1], h->nf[l], ld, false);
+}
+int mi_mlp_get_bgrad(mi_mlp* h, int l, int r, float* dst) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  MI_REQUIRE(r >= 0 && r < h->R, "replica index %d out of range [0,%d)", r, h->R);
+  return download_matrix(h, dst, h->grads + (size_t)r * h->stride + h->boff[l], 1, h->nf[l + 1], h->nf[l + 1], false);
+}
+int mi_mlp_get_dx(mi_mlp* h, float* dst, int ld) {
+  if (int rc = check_handle(h)) return rc;
+  return download_matrix(h, dst, h->dx, h->MB, h->nf[0], ld, h->dtype == MI_BF16);
+}
+
+int mi_mlp_param_count(mi_mlp* h, size_t* params, size_t* replica_stride) {
+  if (int rc = check_handle(h)) return rc;
+  if (params) *params = h->P;
+  if (replica_stride) *replica_stride = h->stride;
+  return MI_OK;
+}
+
+int mi_mlp_enable_timing(mi_mlp* h, int on) {
+  if (int rc = check_handle(h)) return rc;
+  if (!on)
+    if (int rc = harvest(h)) return rc;
+  h->timing = on != 0;
+  return MI_OK;
+}
+int mi_mlp_reset_timings(mi_mlp* h) {
+  if (int rc = check_handle(h)) return rc;
+  if (int rc = harvest(h)) return rc;
+  std::fill(h->ms.begin(), h->ms.end(), 0.0);
+  std::fill(h->launches.begin(), h->launches.end(), 0);
+  return MI_OK;
+}
+int mi_mlp_get_timings(mi_mlp* h, double* ms, long long* launches) {
+  if (int rc = check_handle(h)) return rc;
+  if (int rc = harvest(h)) return rc;
+  if (ms) std::memcpy(ms, h->ms.data(), h->ms.size() * sizeof(double));
+  if (launches) std::memcpy(launches, h->launches.data(), h->launches.size() * sizeof(long long));
+  return MI_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,439 @@
+// fp32 GEMM kernels for gfx950 on v_mfma_f32_32x32x2_f32, one template for the three operand
+// layouts of the MLP step:
+//   NT  C = A[M,K] * B[N,K]^T   forward        (reference call site mlp_omp.cc:474-488)
+//   NN  C = A[M,K] * B[K,N]     input gradient (mlp_omp.cc:657-671)
+//   TN  C = A[K,M]^T * B[K,N]   weight gradient, batched over replicas (mlp_omp.cc:565-580)
+//
+// Structure of one workgroup (WM x WN wavefronts of 64 lanes):
+//   - owns a BM x BN tile of C; walks K in steps of BK;
+//   - global -> registers -> LDS with two LDS buffers, so the loads of step t+1 are in flight
+//     while step t is multiplied (one barrier per step);
+//   - each wavefront owns a (BM/WM) x (BN/WN) sub-tile as TM x TN blocks of 32 x 32 held in
+//     accumulator registers.
+//
+// Operand fragments.  One MFMA consumes, per lane, one A value A[i = lane%32][k = lane/32] and
+// one B value B[k = lane/32][j = lane%32].  A lane fetches four values with one 16-byte LDS
+// read, and what the four values are depends on how the operand lies in memory:
+//   * "K-major" operand (k contiguous: A of NT/NN, B of NT): the tile is stored [row][k] with
+//     a 4-float pad per row; the lane reads k = kk*8 + 4*(lane/32) + {0,1,2,3} of its row and
+//     feeds them to four consecutive MFMAs of the same 32 x 32 block.
+//   * "M-major" operand (rows contiguous: A of TN, B of NN/TN): the tile is stored [k][row];
+//     the lane reads rows TM*(lane%32) + {0..TM-1} of one k and feeds them to the TM blocks of
+//     one MFMA step, i.e. block b of the wavefront owns the interleaved rows TM*i + b.
+// Both choices walk k in the same order (MFMA step q of chunk kk multiplies k = kk*8 + q on
+// lanes 0-31 and kk*8 + 4 + q on lanes 32-63), so any pairing of the two is consistent.
+//
+// Result layout of a 32 x 32 block: lane holds column (lane%32), rows 8*(r/4) + 4*(lane/32) + r%4
+// for accumulator register r = 0..15.
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+namespace mi {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+enum Epilogue { EPI_NONE = 0, EPI_BIAS_RELU = 1, EPI_MASK = 2 };
+
+struct GemmArgs {
+  int M, N, K;
+  const float* A;
+  const float* B;
+  float* C;
+  int lda, ldb, ldc;
+  // batch (blockIdx.z): element offsets added per batch index
+  long long batchA, batchB, batchC;
+  // epilogue
+  const float* bias;  // EPI_BIAS_RELU: [N] or null
+  int relu;           // EPI_BIAS_RELU
+  const float* mask;  // EPI_MASK: [M x N], result zeroed where mask <= 0
+  int ldmask;
+  // tile rasterisation
+  int tiles_m, tiles_n;
+};
+
+// Maps the flat workgroup index to a C tile.  Workgroups are handed to the 8 XCDs round-robin
+// (id % 8) and each XCD has a private L2; giving XCD x the contiguous range
+// [x*T/8, (x+1)*T/8) of the row-major tile order keeps the tiles that share an A panel (same
+// tile row) on one L2.  Falls back to the identity when the tile count is not a multiple of 8.
+__device__ __forceinline__ void tile_of_block(const GemmArgs& p, int& tm, int& tn) {
+  int id = blockIdx.x;
+  const int total = p.tiles_m * p.tiles_n;
+  if ((total & 7) == 0) {
+    const int per_xcd = total >> 3;
+    id = (id & 7) * per_xcd + (id >> 3);
+  }
+  tm = id / p.tiles_n;
+  tn = id - tm * p.tiles_n;
+}
+
+template <int ROWS, int BK, bool KMAJOR>
+struct TileShape {
+  // K-major: [ROWS][BK + 4]; M-major: [BK][ROWS]
+  static constexpr int kStride = KMAJOR ? (BK + 4) : ROWS;
+  static constexpr int kFloats = KMAJOR ? ROWS * (BK + 4) : BK * ROWS;
+  static constexpr int kVecs = ROWS * BK / 4;  // float4 per tile
+};
+
+// Global -> registers for one operand tile.  `base` points at the tile's first element for this
+// K step.  NV = float4 per thread.
+template <int ROWS, int BK, bool KMAJOR, int NT, int NV>
+__device__ __forceinline__ void load_tile(f32x4 (&v)[NV], const float* __restrict__ base, int ld,
+                                          int tid) {
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int idx = tid + i * NT;
+    if (KMAJOR) {
+      const int row = idx / (BK / 4), c4 = idx % (BK / 4);
+      v[i] = *reinterpret_cast<const f32x4*>(base + (size_t)row * ld + c4 * 4);
+    } else {
+      const int k = idx / (ROWS / 4), c4 = idx % (ROWS / 4);
+      v[i] = *reinterpret_cast<const f32x4*>(base + (size_t)k * ld + c4 * 4);
+    }
+  }
+}
+
+template <int ROWS, int BK, bool KMAJOR, int NT, int NV>
+__device__ __forceinline__ void store_tile(float* lds, const f32x4 (&v)[NV], int tid) {
+  using TS = TileShape<ROWS, BK, KMAJOR>;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int idx = tid + i * NT;
+    if (KMAJOR) {
+      const int row = idx / (BK / 4), c4 = idx % (BK / 4);
+      *reinterpret_cast<f32x4*>(lds + row * TS::kStride + c4 * 4) = v[i];
+    } else {
+      const int k = idx / (ROWS / 4), c4 = idx % (ROWS / 4);
+      *reinterpret_cast<f32x4*>(lds + k * TS::kStride + c4 * 4) = v[i];
+    }
+  }
+}
+
+// LDS -> fragment registers for one 8-wide K chunk.  frag[b][q]: value for block b, MFMA step q.
+template <int ROWS, int BK, bool KMAJOR, int TB>
+__device__ __forceinline__ void load_frag(float (&frag)[TB][4], const float* lds, int wave_row0,
+                                          int kk, int lane) {
+  using TS = TileShape<ROWS, BK, KMAJOR>;
+  const int l32 = lane & 31, hi = lane >> 5;
+  if (KMAJOR) {
+#pragma unroll
+    for (int b = 0; b < TB; ++b) {
+      const f32x4 t = *reinterpret_cast<const f32x4*>(lds + (wave_row0 + b * 32 + l32) * TS::kStride +
+                                                      kk * 8 + hi * 4);
+      frag[b][0] = t[0];
+      frag[b][1] = t[1];
+      frag[b][2] = t[2];
+      frag[b][3] = t[3];
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float* src = lds + (kk * 8 + hi * 4 + q) * TS::kStride + wave_row0 + TB * l32;
+      if (TB == 4) {
+        const f32x4 t = *reinterpret_cast<const f32x4*>(src);
+        frag[0][q] = t[0];
+        frag[1 % TB][q] = t[1];
+        frag[2 % TB][q] = t[2];
+        frag[3 % TB][q] = t[3];
+      } else if (TB == 2) {
+        const f32x2 t = *reinterpret_cast<const f32x2*>(src);
+        frag[0][q] = t[0];
+        frag[1 % TB][q] = t[1];
+      } else {
+        frag[0][q] = src[0];
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, int EPI>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int WTM = BM / WM, WTN = BN / WN;  // wavefront sub-tile
+  constexpr int TM = WTM / 32, TN = WTN / 32;  // 32x32 blocks per wavefront
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wavefront tile must be whole 32x32 blocks");
+  static_assert(BK % 8 == 0, "BK must be a multiple of 8");
+  static_assert(A_KMAJOR || TM == 1 || TM == 2 || TM == 4, "interleaved A needs TM in {1,2,4}");
+  static_assert(B_KMAJOR || TN == 1 || TN == 2 || TN == 4, "interleaved B needs TN in {1,2,4}");
+  using TA = TileShape<BM, BK, A_KMAJOR>;
+  using TB = TileShape<BN, BK, B_KMAJOR>;
+  static_assert(TA::kVecs % NT == 0 && TB::kVecs % NT == 0, "tile must divide over the threads");
+  constexpr int NVA = TA::kVecs / NT, NVB = TB::kVecs / NT;
+
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  // LDS layout: [A buffer 0][A buffer 1][B buffer 0][B buffer 1]
+  auto As = [&](int buf) { return smem + buf * TA::kFloats; };
+  auto Bs = [&](int buf) { return smem + 2 * TA::kFloats + buf * TB::kFloats; };
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
+
+  int tile_m, tile_n;
+  tile_of_block(p, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const float* __restrict__ A = p.A + (size_t)blockIdx.z * p.batchA;
+  const float* __restrict__ B = p.B + (size_t)blockIdx.z * p.batchB;
+  float* __restrict__ C = p.C + (size_t)blockIdx.z * p.batchC;
+
+  // first element of this workgroup's panel, and the pointer advance per K step
+  const float* a_ptr = A_KMAJOR ? A + (size_t)m0 * p.lda : A + m0;
+  const float* b_ptr = B_KMAJOR ? B + (size_t)n0 * p.ldb : B + n0;
+  const size_t a_step = A_KMAJOR ? (size_t)BK : (size_t)BK * p.lda;
+  const size_t b_step = B_KMAJOR ? (size_t)BK : (size_t)BK * p.ldb;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  f32x4 ra[NVA], rb[NVB];
+  load_tile<BM, BK, A_KMAJOR, NT, NVA>(ra, a_ptr, p.lda, tid);
+  load_tile<BN, BK, B_KMAJOR, NT, NVB>(rb, b_ptr, p.ldb, tid);
+  store_tile<BM, BK, A_KMAJOR, NT, NVA>(As(0), ra, tid);
+  store_tile<BN, BK, B_KMAJOR, NT, NVB>(Bs(0), rb, tid);
+  __syncthreads();
+
+  const int nk = p.K / BK;
+  for (int t = 0; t < nk; ++t) {
+    const int cur = t & 1;
+    if (t + 1 < nk) {
+      a_ptr += a_step;
+      b_ptr += b_step;
+      load_tile<BM, BK, A_KMAJOR, NT, NVA>(ra, a_ptr, p.lda, tid);
+      load_tile<BN, BK, B_KMAJOR, NT, NVB>(rb, b_ptr, p.ldb, tid);
+    }
+
+#pragma unroll
+    for (int kk = 0; kk < BK / 8; ++kk) {
+      float fa[TM][4], fb[TN][4];
+      load_frag<BM, BK, A_KMAJOR, TM>(fa, As(cur), wm0, kk, lane);
+      load_frag<BN, BK, B_KMAJOR, TN>(fb, Bs(cur), wn0, kk, lane);
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q], acc[i][j], 0, 0, 0);
+    }
+
+    if (t + 1 < nk) {
+      store_tile<BM, BK, A_KMAJOR, NT, NVA>(As(cur ^ 1), ra, tid);
+      store_tile<BN, BK, B_KMAJOR, NT, NVB>(Bs(cur ^ 1), rb, tid);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: registers -> global, fused bias/ReLU or ReLU mask --------------------------
+  const int l32 = lane & 31, hi = lane >> 5;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int rb32 = 8 * (r >> 2) + 4 * hi + (r & 3);  // row inside the 32x32 block
+      const int row = m0 + wm0 + (A_KMAJOR ? i * 32 + rb32 : TM * rb32 + i);
+      float* crow = C + (size_t)row * p.ldc;
+      if (B_KMAJOR) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int col = n0 + wn0 + j * 32 + l32;
+          float v = acc[i][j][r];
+          if (EPI == EPI_BIAS_RELU) {
+            if (p.bias) v += p.bias[col];
+            if (p.relu) v = v > 0.0f ? v : 0.0f;
+          } else if (EPI == EPI_MASK) {
+            if (!(p.mask[(size_t)row * p.ldmask + col] > 0.0f)) v = 0.0f;
+          }
+          crow[col] = v;
+        }
+      } else {
+        // interleaved columns: this lane owns TN consecutive columns -> one vector store
+        const int col = n0 + wn0 + TN * l32;
+        float v[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
+        if (EPI == EPI_BIAS_RELU) {
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            if (p.bias) v[j] += p.bias[col + j];
+            if (p.relu) v[j] = v[j] > 0.0f ? v[j] : 0.0f;
+          }
+        } else if (EPI == EPI_MASK) {
+          const float* mrow = p.mask + (size_t)row * p.ldmask + col;
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            if (!(mrow[j] > 0.0f)) v[j] = 0.0f;
+        }
+        if (TN == 4) {
+          f32x4 o = {v[0], v[1 % TN], v[2 % TN], v[3 % TN]};
+          *reinterpret_cast<f32x4*>(crow + col) = o;
+        } else if (TN == 2) {
+          f32x2 o = {v[0], v[1 % TN]};
+          *reinterpret_cast<f32x2*>(crow + col) = o;
+        } else {
+          crow[col] = v[0];
+        }
+      }
+    }
+  }
+}
+
+// ---- any-shape fallback ----------------------------------------------------------------------
+// Plain LDS-tiled SIMT kernel with fully guarded loads and stores; used when a dimension is not
+// a multiple of the MFMA tile or a pointer / leading dimension is not 16-byte aligned.
+// 16 x 16 threads, each computing a 4 x 4 patch of a 64 x 64 tile.
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
+__global__ __launch_bounds__(256) void gemm_f32_generic(GemmArgs p) {
+  constexpr int T = 64, KS = 16;
+  __shared__ float As[KS][T + 1];
+  __shared__ float Bs[KS][T + 1];
+  const float* __restrict__ A = p.A + (size_t)blockIdx.z * p.batchA;
+  const float* __restrict__ B = p.B + (size_t)blockIdx.z * p.batchB;
+  float* __restrict__ C = p.C + (size_t)blockIdx.z * p.batchC;
+  const int m0 = blockIdx.y * T, n0 = blockIdx.x * T;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < p.K; k0 += KS) {
+    for (int e = threadIdx.x; e < T * KS; e += 256) {
+      int r, k;
+      if (A_KMAJOR) { r = e / KS; k = e % KS; } else { k = e / T; r = e % T; }
+      const int gm = m0 + r, gk = k0 + k;
+      float v = 0.0f;
+      if (gm < p.M && gk < p.K) v = A_KMAJOR ? A[(size_t)gm * p.lda + gk] : A[(size_t)gk * p.lda + gm];
+      As[k][r] = v;
+      if (B_KMAJOR) { r = e / KS; k = e % KS; } else { k = e / T; r = e % T; }
+      const int gn = n0 + r;
+      v = 0.0f;
+      if (gn < p.N && gk < p.K) v = B_KMAJOR ? B[(size_t)gn * p.ldb + gk] : B[(size_t)gk * p.ldb + gn];
+      Bs[k][r] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = Bs[k][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = m0 + ty * 4 + i;
+    if (row >= p.M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int col = n0 + tx * 4 + j;
+      if (col >= p.N) continue;
+      float v = acc[i][j];
+      if (EPI == EPI_BIAS_RELU) {
+        if (p.bias) v += p.bias[col];
+        if (p.relu) v = v > 0.0f ? v : 0.0f;
+      } else if (EPI == EPI_MASK) {
+        if (!(p.mask[(size_t)row * p.ldmask + col] > 0.0f)) v = 0.0f;
+      }
+      C[(size_t)row * p.ldc + col] = v;
+    }
+  }
+}
+
+// ---- launch ------------------------------------------------------------------------------------
+
+template <int BM, int BN, int BK, int WM, int WN, bool AK, bool BKM, int EPI>
+static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
+  using TA = TileShape<BM, BK, AK>;
+  using TB = TileShape<BN, BK, BKM>;
+  constexpr size_t lds_bytes = 2 * (TA::kFloats + TB::kFloats) * sizeof(float);
+  auto kern = gemm_f32_mfma<BM, BN, BK, WM, WN, AK, BKM, EPI>;
+  static bool attr_set = false;  // opt in to more than 64 KiB of dynamic LDS once per kernel
+  if (lds_bytes > 64 * 1024 && !attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  p.tiles_m = p.M / BM;
+  p.tiles_n = p.N / BN;
+  dim3 grid(p.tiles_m * p.tiles_n, 1, batch);
+  hipLaunchKernelGGL(kern, grid, dim3(WM * WN * 64), lds_bytes, s, p);
+  return hipGetLastError();
+}
+
+template <bool AK, bool BKM, int EPI>
+static hipError_t launch_generic(GemmArgs& p, int batch, hipStream_t s) {
+  dim3 grid((p.N + 63) / 64, (p.M + 63) / 64, batch);
+  hipLaunchKernelGGL((gemm_f32_generic<AK, BKM, EPI>), grid, dim3(256), 0, s, p);
+  return hipGetLastError();
+}
+
+static inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
+
+// Picks a tile configuration.  `variant` (0 = automatic) lets the tuning harness force one.
+template <bool AK, bool BKM, int EPI>
+static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant) {
+  if (p.M <= 0 || p.N <= 0 || batch <= 0) return hipSuccess;
+  const bool vec_ok = aligned16(p.A) && aligned16(p.B) && aligned16(p.C) && p.lda % 4 == 0 &&
+                      p.ldb % 4 == 0 && p.ldc % 4 == 0 && p.batchA % 4 == 0 && p.batchB % 4 == 0 &&
+                      p.batchC % 4 == 0 && p.K > 0;
+  auto fits = [&](int bm, int bn, int bk) { return vec_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0; };
+  if (variant == 0) {
+    // automatic choice: the largest tile that still yields at least one workgroup per CU
+    const long long tiles128 = (long long)(p.M / 128) * (p.N / 128) * batch;
+    if (fits(256, 128, 32) && (long long)(p.M / 256) * (p.N / 128) * batch >= 512) variant = 3;
+    else if (fits(128, 128, 32) && tiles128 >= 128) variant = 1;
+    else if (fits(64, 64, 32)) variant = 4;
+    else variant = -1;
+  }
+  switch (variant) {
+    case 1: if (fits(128, 128, 32)) return launch_mfma<128, 128, 32, 2, 2, AK, BKM, EPI>(p, batch, s); break;
+    case 2: if (fits(128, 128, 32)) return launch_mfma<128, 128, 32, 2, 4, AK, BKM, EPI>(p, batch, s); break;
+    case 3: if (fits(256, 128, 32)) return launch_mfma<256, 128, 32, 2, 2, AK, BKM, EPI>(p, batch, s); break;
+    case 4: if (fits(64, 64, 32)) return launch_mfma<64, 64, 32, 2, 2, AK, BKM, EPI>(p, batch, s); break;
+    case 5: if (fits(128, 128, 16)) return launch_mfma<128, 128, 16, 2, 2, AK, BKM, EPI>(p, batch, s); break;
+    case 6: if (fits(256, 128, 16)) return launch_mfma<256, 128, 16, 4, 2, AK, BKM, EPI>(p, batch, s); break;
+    case 7: if (fits(128, 64, 32)) return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI>(p, batch, s); break;
+    default: break;
+  }
+  return launch_generic<AK, BKM, EPI>(p, batch, s);
+}
+
+hipError_t sgemm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                    int ldc, const float* bias, int relu, hipStream_t s, int variant) {
+  GemmArgs p{};
+  p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+  p.bias = bias; p.relu = relu;
+  return dispatch<true, true, EPI_BIAS_RELU>(p, 1, s, variant);
+}
+
+hipError_t sgemm_nn(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
+                    int ldc, const float* mask, int ldmask, hipStream_t s, int variant) {
+  GemmArgs p{};
+  p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+  p.mask = mask; p.ldmask = ldmask;
+  if (mask) return dispatch<true, false, EPI_MASK>(p, 1, s, variant);
+  return dispatch<true, false, EPI_NONE>(p, 1, s, variant);
+}
+
+hipError_t sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
+                    float* C, int ldc, long long strideC, hipStream_t s, int variant) {
+  GemmArgs p{};
+  p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+  p.batchA = (long long)K * lda;  // replica r reads rows [r*K, (r+1)*K) of both operands
+  p.batchB = (long long)K * ldb;
+  p.batchC = strideC;
+  return dispatch<false, false, EPI_NONE>(p, R, s, variant);
+}
+
+}  // namespace mi

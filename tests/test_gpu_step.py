@@ -1,0 +1,137 @@
+"""GPU parity of the whole training step (handle API of the C ABI) against the CPU oracle on
+identical seeded inputs.  Bound: rel-err <= 1e-4 on Y, dX, dW/db and the updated W/b."""
+import numpy as np
+import pytest
+
+import oracle
+from conftest import FP32_TOL, rel_err
+from tbb_test_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+LR = 0.01
+
+
+def build(nf, B, R, seed, flags=0, bias_scale=0.0):
+    X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed)
+    if bias_scale:
+        rng = np.random.default_rng(seed)
+        bs = [(bias_scale * rng.standard_normal(b.shape)).astype(np.float32) for b in bs]
+    h = capi.MlpHandle(nf, B, R, flags=flags)
+    for l in range(len(nf) - 1):
+        h.set_weights(l, Ws[l], bs[l])
+    h.set_input(X)
+    h.set_dy(dY)
+    return h, (X, Ws, bs, dY)
+
+
+def compare_step(h, ref, nf, R, tol=FP32_TOL):
+    L = len(nf) - 1
+    for l in range(L + 1):
+        assert rel_err(h.activation(l), ref.acts[l]) <= tol, f"activation {l}"
+    assert rel_err(h.dx(), ref.dX) <= tol, "dX"
+    for l in range(L):
+        for r in range(R):
+            assert rel_err(h.wgrad_of(l, r), ref.dW[r][l]) <= tol, f"dW layer {l} replica {r}"
+            assert rel_err(h.bgrad_of(l, r), ref.db[r][l]) <= tol, f"db layer {l} replica {r}"
+        assert rel_err(h.weight(l), ref.W_new[l]) <= tol, f"updated W {l}"
+        assert rel_err(h.bias(l), ref.b_new[l]) <= tol, f"updated b {l}"
+
+
+CONFIGS = {
+    # name: (nfeatures, batch per replica, R)
+    "C1_tiny": ([512, 512, 512, 512], 256, 2),           # benchmark config 1
+    "rect": ([256, 384, 128, 640], 128, 3),              # rectangular layers, odd replica count
+    "ragged": ([100, 70, 33, 1], 37, 2),                 # nothing is a tile multiple; last layer N = 1
+    "single_replica": ([128, 128], 64, 1),               # R = 1: the reduce degenerates to plain SGD
+}
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+@pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, capi.FLAG_NO_GRAPH | capi.FLAG_RELU_LAST,
+                                   capi.FLAG_NO_GRAPH | capi.FLAG_PER_LAYER_UPDATE])
+def test_step_matches_oracle(name, flags):
+    nf, B, R = CONFIGS[name]
+    h, (X, Ws, bs, dY) = build(nf, B, R, seed=2024, flags=flags, bias_scale=0.1)
+    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR, relu_last=bool(flags & capi.FLAG_RELU_LAST))
+    h.step(LR)
+    h.sync()
+    compare_step(h, ref, nf, R)
+    h.close()
+
+
+def test_per_operation_entry_points_match_step():
+    """Driving the step through mi_fc_forward / wgrad / dgrad / mi_reduce_sgd gives the same
+    bits as mi_mlp_step."""
+    nf, B, R = CONFIGS["rect"]
+    h1, _ = build(nf, B, R, seed=7, flags=capi.FLAG_NO_GRAPH)
+    h2, _ = build(nf, B, R, seed=7, flags=capi.FLAG_NO_GRAPH)
+    h1.step(LR)
+    L = len(nf) - 1
+    for l in range(L):
+        h2.forward(l)
+    for l in reversed(range(L)):
+        h2.wgrad(l)
+        h2.dgrad(l)
+    h2.reduce_sgd(LR)
+    for l in range(L):
+        assert np.array_equal(h1.weight(l), h2.weight(l))
+        assert np.array_equal(h1.bias(l), h2.bias(l))
+    assert np.array_equal(h1.dx(), h2.dx())
+    h1.close(); h2.close()
+
+
+def test_graph_replay_matches_eager_over_several_steps():
+    """mi_mlp_step replays a captured HIP graph from the second call on; every replay must give
+    the bits of the eager schedule, with host synchronisation and downloads between replays."""
+    nf, B, R = CONFIGS["C1_tiny"]
+    hg, _ = build(nf, B, R, seed=11, flags=0)
+    he, _ = build(nf, B, R, seed=11, flags=capi.FLAG_NO_GRAPH)
+    for step in range(6):
+        hg.step(LR)
+        he.step(LR)
+        hg.sync(); he.sync()
+        for l in range(len(nf) - 1):
+            assert np.array_equal(hg.weight(l), he.weight(l)), (step, l)
+        assert np.array_equal(hg.dx(), he.dx()), step
+    hg.close(); he.close()
+
+
+def test_multi_step_training_tracks_oracle():
+    """Three consecutive steps (weights feed back into the next forward) stay within tolerance."""
+    nf, B, R = [256, 256, 256], 128, 2
+    h, (X, Ws, bs, dY) = build(nf, B, R, seed=5, flags=0)
+    for _ in range(3):
+        ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR)
+        Ws, bs = [w.copy() for w in ref.W_new], [b.copy() for b in ref.b_new]
+        h.step(LR)
+    h.sync()
+    for l in range(2):
+        assert rel_err(h.weight(l), Ws[l]) <= FP32_TOL
+    h.close()
+
+
+def test_timing_slots_are_filled():
+    nf, B, R = CONFIGS["C1_tiny"]
+    h, _ = build(nf, B, R, seed=1)
+    h.enable_timing(True)
+    for _ in range(2):
+        h.step(LR)
+    ms, cnt = h.timings()
+    L = len(nf) - 1
+    assert np.all(cnt[0] == 2) and np.all(cnt[1] == 2) and np.all(cnt[2] == 2)  # fwd, wgt_grad, bwd
+    assert cnt[3, 0] == 2 and np.all(cnt[3, 1:] == 0)  # one all-layer update per step, booked on layer 0
+    assert np.all(ms[:3] > 0) and ms[3, 0] > 0
+    assert np.all(ms[4:] == 0)
+    h.close()
+
+
+def test_benchmark_config_2_full_size():
+    """Benchmark config 2 (8 x 1024, batch 1024 x 4 replicas) at full size against the oracle."""
+    nf, B, R = [1024] * 9, 1024, 4
+    h, (X, Ws, bs, dY) = build(nf, B, R, seed=42)
+    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR)
+    h.step(LR)
+    h.sync()
+    compare_step(h, ref, nf, R)
+    h.close()
