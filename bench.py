@@ -1,0 +1,166 @@
+#!/usr/bin/env python3
+"""Benchmark of the MLP training step (forward, backward, gradient reduce + SGD) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C2]
+
+A "step" is one pass of the whole hot path over one batch of seeded synthetic input: L forward
+GEMMs, L weight-gradient GEMMs (R replicas each), L bias gradients, L input-gradient GEMMs and
+the R-way gradient reduce with the SGD update.  Inputs and weights are resident in HBM before
+the timed region starts.  Every timed step starts from the initial weights (a device-to-device
+restore that is inside the timed region), so that values stay finite however many sum-reduced
+SGD steps are run.
+
+Prints one JSON line:
+  value          whole-step throughput, TFLOP/s on the reference's FLOP model
+                 3 * 2 * (R*B) * sum_l N_l*N_{l+1}   (mlp_omp.cc:492,584,675)
+  ms_per_step    wall clock of the timed loop / K
+  roofline       the GEMM kernels (the dominant kernels): FLOP per launch / average launch
+                 duration from HIP events on the launching stream, against the fp32 MFMA peak
+  roofline_reduce  the reduce+SGD kernel: (R+2)*4*P bytes / its launch duration, against HBM peak
+  cpu_baseline   the CPU restatement of the reference's mlp_omp timed on this host's cores
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+CONFIGS = {
+    # name: (layers, width, batch per replica, replicas, dtype)
+    "C1": (3, 512, 256, 2, "f32"),
+    "C2": (8, 1024, 1024, 4, "f32"),
+    "C3": (4, 4096, 2048, 2, "f32"),
+    "C4": (20, 2048, 256, 8, "f32"),
+    "C5": (8, 8192, 4096, 4, "bf16"),
+}
+PEAK_TFLOPS = {"f32": 157.3, "bf16": 2516.6}  # MI355X dense MFMA peaks
+PEAK_HBM_GBPS = 8000.0
+METRIC = "MLP fwd+bwd+reduce step ms & TFLOP/s on 1 MI355X; grad-reduce GB/s"
+
+
+def cpu_baseline(nf, B, R, lr, budget_s):
+    """Times the CPU restatement of the reference path on this host (rank 0, N = 1 only)."""
+    import oracle
+    from oracle import cpu_baseline as port
+
+    return port.run(nf, B, R, lr, budget_s)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
+    ap.add_argument("--lr", type=float, default=0.01)
+    ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--overlap", action="store_true", help="per-layer update on a second stream")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg (0 = skip)")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; there is no multi-GPU path (no collectives). "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+
+    from tbb_test_amd import capi, hostlib
+
+    layers, width, B, R, dtype = CONFIGS[args.config]
+    nf = [width] * (layers + 1)
+    info = capi.device_info()
+
+    X, Ws, dY = hostlib.init_problem(nf, B, R, args.seed)
+    flags = capi.FLAG_PER_LAYER_UPDATE if args.overlap else 0
+    h = capi.MlpHandle(nf, B, R, dtype=capi.MI_BF16 if dtype == "bf16" else capi.MI_F32, flags=flags)
+    for l in range(layers):
+        h.set_weights(l, Ws[l], None)
+    h.set_input(X)
+    h.set_dy(dY)
+    h.snapshot_weights()
+    params, _ = h.param_count()
+
+    def one_step():
+        h.restore_weights()
+        h.step(args.lr)
+
+    for _ in range(args.warmup):
+        one_step()
+    h.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        one_step()
+    h.sync()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+
+    # per-kernel durations: same loop again with a HIP event pair around every launch
+    h.enable_timing(True)
+    h.reset_timings()
+    for _ in range(args.steps):
+        one_step()
+    ms, cnt = h.timings()
+    h.enable_timing(False)
+    finite = all(bool(np.isfinite(h.weight(l)).all()) for l in range(layers))
+    h.close()
+
+    rows = R * B
+    flop_per_gemm = 2.0 * rows * width * width          # every GEMM launch of a square model
+    gemm_flop_step = 3 * layers * flop_per_gemm
+    gemm_ms = float(ms[0:3].sum())
+    gemm_launches = int(cnt[0:3].sum())
+    gemm_avg_ms = gemm_ms / gemm_launches
+    gemm_tflops = flop_per_gemm / (gemm_avg_ms * 1e-3) / 1e12
+    per_phase = {capi.BREAKDOWN_NAMES[i]: float(ms[i].sum() / args.steps) for i in range(4)}
+
+    upd_launches = int(cnt[3].sum())
+    upd_ms = float(ms[3].sum()) / upd_launches
+    # one launch covers all layers unless the per-layer schedule is on
+    upd_bytes = (R + 2) * 4.0 * params * (1 if not args.overlap else 1.0 / layers)
+    if dtype == "bf16":
+        upd_bytes += 2.0 * params * (1 if not args.overlap else 1.0 / layers)
+    upd_gbps = upd_bytes / (upd_ms * 1e-3) / 1e9
+
+    peak = PEAK_TFLOPS[dtype]
+    out = {
+        "metric": METRIC,
+        "value": round(gemm_flop_step / (ms_per_step * 1e-3) / 1e12, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype,
+        "data": "synthetic",
+        "config": {"workload": f"{args.config}: {layers} FC layers of width {width}, ReLU between layers, "
+                               f"batch {B} per replica x {R} replicas, lr {args.lr}, seed {args.seed}",
+                   "schedule": "per-layer update on a second stream" if args.overlap else "one update launch",
+                   "device": info["name"], "num_cus": info["num_cus"]},
+        "gemm_flop_per_step": gemm_flop_step,
+        "phase_ms_per_step": {k: round(v, 4) for k, v in per_phase.items()},
+        "gemm_tflops": round(gemm_tflops, 2),
+        "reduce_gbps": round(upd_gbps, 1),
+        "weights_finite": finite,
+        "roofline": {"kernel": "gemm_f32_mfma (nt, nn, tn)" if dtype == "f32" else "gemm_bf16_mfma",
+                     "bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(gemm_tflops / peak, 4), "traffic": None,
+                     "flop_per_launch": flop_per_gemm, "avg_launch_us": round(gemm_avg_ms * 1e3, 2),
+                     "launches": gemm_launches},
+        "roofline_reduce": {"kernel": "reduce_sgd_vec4", "bound": "hbm", "achieved": round(upd_gbps, 1),
+                            "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(upd_gbps / PEAK_HBM_GBPS, 4),
+                            "traffic": None, "bytes_per_launch": upd_bytes, "avg_launch_us": round(upd_ms * 1e3, 2)},
+    }
+    if args.cpu_seconds > 0:
+        out["cpu_baseline"] = cpu_baseline(nf, B, R, args.lr, args.cpu_seconds)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -196,6 +196,13 @@ int mi_mlp_get_wgrad(mi_mlp* h, int l, int r, float* dst, int ld);
 int mi_mlp_get_bgrad(mi_mlp* h, int l, int r, float* dst);
 int mi_mlp_get_dx(mi_mlp* h, float* dst, int ld);
 
+/* Device-side copy of all weights and biases (snapshot) and its inverse (restore), both
+ * asynchronous on the handle's stream.  A benchmark loop restores before every step so that the
+ * values stay finite over any number of sum-reduced SGD steps; the reference gets the same effect
+ * by benchmarking with alpha = 1e-10 (mlp_omp.cc:609,699,718). */
+int mi_mlp_snapshot_weights(mi_mlp* h);
+int mi_mlp_restore_weights(mi_mlp* h);
+
 /* Number of parameters P = sum_l (N_l*N_{l+1} + N_{l+1}) and the padded element stride between
  * consecutive replicas' gradient arenas. */
 int mi_mlp_param_count(mi_mlp* h, size_t* params, size_t* replica_stride);

@@ -31,7 +31,7 @@ def _load():
         lib.oracle_fc_wgrad.argtypes = [_ci, _ci, _ci, _vp, _ci, _vp, _ci, _vp, _ci, _vp]
         lib.oracle_fc_dgrad.argtypes = [_ci, _ci, _ci, _vp, _ci, _vp, _ci, _vp, _ci, _vp, _ci]
         lib.oracle_reduce_sgd.argtypes = [_vp, _vp, ctypes.c_size_t, ctypes.c_size_t, _ci, ctypes.c_float]
-        lib.oracle_mlp_step.argtypes = [_ci, ctypes.POINTER(_ci), _ci, _ci, _ci, ctypes.c_float, _vp, _vp, _vp, _vp,
+        lib.oracle_mlp_step.argtypes = [_ci, ctypes.POINTER(_ci), _ci, _ci, _ci, _ci, ctypes.c_float, _vp, _vp, _vp, _vp,
                                         _vp, _vp]
         lib.oracle_mlp_step.restype = _ci
         for fn in (lib.oracle_fc_forward, lib.oracle_fc_wgrad, lib.oracle_fc_dgrad, lib.oracle_reduce_sgd):
@@ -100,19 +100,24 @@ class StepResult:
     pass
 
 
-def mlp_step(nf, B, R, X, dY, Ws, bs, lr, relu_last=False):
+def mlp_step(nf, B, R, X, dY, Ws, bs, lr, relu_last=False, given_acts=None):
     """Runs one full step.  Ws[l]: [nf[l+1], nf[l]], bs[l]: [nf[l+1]].
-    Returns an object with acts (list of L+1 arrays), dW[r][l], db[r][l], dX, W_new[l], b_new[l]."""
+    Returns an object with acts (list of L+1 arrays), dW[r][l], db[r][l], dX, W_new[l], b_new[l].
+    given_acts (list of L+1 arrays): skip the forward pass and run the backward pass on these."""
     L = len(nf) - 1
     MB = R * B
     flat = np.concatenate([np.concatenate([_c(Ws[l]).ravel(), _c(bs[l]).ravel()]) for l in range(L)])
     P = flat.size
-    acts = np.empty(sum(MB * n for n in nf), dtype=_f32)
+    if given_acts is None:
+        acts = np.empty(sum(MB * n for n in nf), dtype=_f32)
+    else:
+        acts = np.concatenate([_c(a).ravel() for a in given_acts])
+        assert acts.size == sum(MB * n for n in nf)
     dWall = np.empty(R * P, dtype=_f32)
     dX = np.empty((MB, nf[0]), dtype=_f32)
     X, dY = _c(X), _c(dY)
     arr = (_ci * len(nf))(*nf)
-    rc = _load().oracle_mlp_step(L, arr, B, R, int(relu_last), lr, _p(X), _p(dY), _p(flat), _p(acts), _p(dWall),
+    rc = _load().oracle_mlp_step(L, arr, B, R, int(relu_last), int(given_acts is not None), lr, _p(X), _p(dY), _p(flat), _p(acts), _p(dWall),
                                  _p(dX))
     if rc != 0:
         raise MemoryError("oracle_mlp_step failed")

@@ -118,10 +118,14 @@ void oracle_reduce_sgd(float* W, const float* G, size_t n, size_t stride, int R,
  *   dX  [R*B x nf[0]]
  * relu_last != 0 applies ReLU after the last layer as well (mlp_caffe2.py:215-217 does);
  * the benchmark configs use ReLU between layers only.
+ * given_acts != 0 skips the forward pass and takes `acts` as input: the backward pass is then
+ * evaluated on exactly those activations.  Tests use it to compare a device backward pass on the
+ * device's own activations, because the ReLU mask [A > 0] is discontinuous: an activation that
+ * rounds to +1e-9 on one side and to 0 on the other legitimately flips a whole gradient entry.
  * Returns 0, or -1 on allocation failure.
  */
-int oracle_mlp_step(int L, const int* nf, int B, int R, int relu_last, float lr, const float* X,
-                    const float* dY, float* W, float* acts, float* dWall, float* dX) {
+int oracle_mlp_step(int L, const int* nf, int B, int R, int relu_last, int given_acts, float lr,
+                    const float* X, const float* dY, float* W, float* acts, float* dWall, float* dX) {
   const int MB = R * B;
   size_t P = 0, maxw = 0;
   for (int l = 0; l < L; ++l) P += (size_t)nf[l + 1] * nf[l] + nf[l + 1];
@@ -138,8 +142,8 @@ int oracle_mlp_step(int L, const int* nf, int B, int R, int relu_last, float lr,
   aoff[0] = 0;
   for (int l = 0; l <= L; ++l) aoff[l + 1] = aoff[l] + (size_t)MB * nf[l];
 
-  memcpy(acts, X, sizeof(float) * MB * nf[0]);
-  for (int l = 0; l < L; ++l) {
+  if (!given_acts) memcpy(acts, X, sizeof(float) * MB * nf[0]);
+  for (int l = 0; l < L && !given_acts; ++l) {
     const float* Wl = W + woff[l];
     const float* bl = Wl + (size_t)nf[l + 1] * nf[l];
     int relu = (l < L - 1) || relu_last;

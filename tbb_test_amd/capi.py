@@ -70,6 +70,8 @@ SIGNATURES = {
     "mi_mlp_get_wgrad": [c_void_p, c_int, c_int, c_void_p, c_int],
     "mi_mlp_get_bgrad": [c_void_p, c_int, c_int, c_void_p],
     "mi_mlp_get_dx": [c_void_p, c_void_p, c_int],
+    "mi_mlp_snapshot_weights": [c_void_p],
+    "mi_mlp_restore_weights": [c_void_p],
     "mi_mlp_param_count": [c_void_p, POINTER(c_size_t), POINTER(c_size_t)],
     "mi_mlp_enable_timing": [c_void_p, c_int],
     "mi_mlp_reset_timings": [c_void_p],
@@ -222,6 +224,9 @@ class MlpHandle:
     def wgrad_of(self, l, r): return self._get(lib().mi_mlp_get_wgrad, (self.nf[l + 1], self.nf[l]), l, r)
     def bgrad_of(self, l, r): return self._get(lib().mi_mlp_get_bgrad, (self.nf[l + 1],), l, r)
     def dx(self): return self._get(lib().mi_mlp_get_dx, (self.MB, self.nf[0]))
+
+    def snapshot_weights(self): check(lib().mi_mlp_snapshot_weights(self._h))
+    def restore_weights(self): check(lib().mi_mlp_restore_weights(self._h))
 
     def param_count(self):
         p, s = c_size_t(), c_size_t()

@@ -64,6 +64,8 @@ struct mi_mlp {
   float* params = nullptr;    // [stride]
   float* grads = nullptr;     // [R * stride]
   uint16_t* params16 = nullptr;  // bf16 copy of params (dtype bf16)
+  float* params_saved = nullptr;    // snapshot of params (mi_mlp_snapshot_weights)
+  uint16_t* params16_saved = nullptr;
   std::vector<void*> acts;    // L+1 buffers [MB x nf[l]], fp32 or bf16
   void* dy = nullptr;         // upstream gradient [MB x nf[L]]
   void* dz[2] = {nullptr, nullptr};  // gradient ping-pong [MB x max width]
@@ -569,6 +571,8 @@ int mi_mlp_destroy(mi_mlp* h) {
   (void)hipFree(h->params);
   (void)hipFree(h->grads);
   (void)hipFree(h->params16);
+  (void)hipFree(h->params_saved);
+  (void)hipFree(h->params16_saved);
   for (void* a : h->acts) (void)hipFree(a);
   (void)hipFree(h->dy);
   (void)hipFree(h->dz[0]);
@@ -698,6 +702,26 @@ int mi_mlp_get_bgrad(mi_mlp* h, int l, int r, float* dst) {
 int mi_mlp_get_dx(mi_mlp* h, float* dst, int ld) {
   if (int rc = check_handle(h)) return rc;
   return download_matrix(h, dst, h->dx, h->MB, h->nf[0], ld, h->dtype == MI_BF16);
+}
+
+int mi_mlp_snapshot_weights(mi_mlp* h) {
+  if (int rc = check_handle(h)) return rc;
+  if (!h->params_saved) MI_HIP(hipMalloc((void**)&h->params_saved, h->stride * 4));
+  MI_HIP(hipMemcpyAsync(h->params_saved, h->params, h->stride * 4, hipMemcpyDeviceToDevice, h->stream));
+  if (h->params16) {
+    if (!h->params16_saved) MI_HIP(hipMalloc((void**)&h->params16_saved, h->stride * 2));
+    MI_HIP(hipMemcpyAsync(h->params16_saved, h->params16, h->stride * 2, hipMemcpyDeviceToDevice, h->stream));
+  }
+  return MI_OK;
+}
+
+int mi_mlp_restore_weights(mi_mlp* h) {
+  if (int rc = check_handle(h)) return rc;
+  MI_REQUIRE(h->params_saved != nullptr, "no snapshot taken");
+  MI_HIP(hipMemcpyAsync(h->params, h->params_saved, h->stride * 4, hipMemcpyDeviceToDevice, h->stream));
+  if (h->params16)
+    MI_HIP(hipMemcpyAsync(h->params16, h->params16_saved, h->stride * 2, hipMemcpyDeviceToDevice, h->stream));
+  return MI_OK;
 }
 
 int mi_mlp_param_count(mi_mlp* h, size_t* params, size_t* replica_stride) {

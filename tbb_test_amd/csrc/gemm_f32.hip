@@ -304,14 +304,14 @@ __global__ __launch_bounds__(256) void gemm_f32_generic(GemmArgs p) {
     for (int e = threadIdx.x; e < T * KS; e += 256) {
       int r, k;
       if (A_KMAJOR) { r = e / KS; k = e % KS; } else { k = e / T; r = e % T; }
-      const int gm = m0 + r, gk = k0 + k;
+      const int gm = m0 + r, gka = k0 + k;
       float v = 0.0f;
-      if (gm < p.M && gk < p.K) v = A_KMAJOR ? A[(size_t)gm * p.lda + gk] : A[(size_t)gk * p.lda + gm];
+      if (gm < p.M && gka < p.K) v = A_KMAJOR ? A[(size_t)gm * p.lda + gka] : A[(size_t)gka * p.lda + gm];
       As[k][r] = v;
       if (B_KMAJOR) { r = e / KS; k = e % KS; } else { k = e / T; r = e % T; }
-      const int gn = n0 + r;
+      const int gn = n0 + r, gkb = k0 + k;
       v = 0.0f;
-      if (gn < p.N && gk < p.K) v = B_KMAJOR ? B[(size_t)gn * p.ldb + gk] : B[(size_t)gk * p.ldb + gn];
+      if (gn < p.N && gkb < p.K) v = B_KMAJOR ? B[(size_t)gn * p.ldb + gkb] : B[(size_t)gkb * p.ldb + gn];
       Bs[k][r] = v;
     }
     __syncthreads();

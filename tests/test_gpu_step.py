@@ -25,9 +25,13 @@ def build(nf, B, R, seed, flags=0, bias_scale=0.0):
     return h, (X, Ws, bs, dY)
 
 
-def compare_step(h, ref, nf, R, tol=FP32_TOL):
+def bits_equal(a, b):
+    return np.array_equal(np.asarray(a).view(np.uint32), np.asarray(b).view(np.uint32))
+
+
+def compare_step(h, ref, nf, R, tol=FP32_TOL, forward=True):
     L = len(nf) - 1
-    for l in range(L + 1):
+    for l in range(L + 1 if forward else 0):
         assert rel_err(h.activation(l), ref.acts[l]) <= tol, f"activation {l}"
     assert rel_err(h.dx(), ref.dX) <= tol, "dX"
     for l in range(L):
@@ -75,9 +79,9 @@ def test_per_operation_entry_points_match_step():
         h2.dgrad(l)
     h2.reduce_sgd(LR)
     for l in range(L):
-        assert np.array_equal(h1.weight(l), h2.weight(l))
-        assert np.array_equal(h1.bias(l), h2.bias(l))
-    assert np.array_equal(h1.dx(), h2.dx())
+        assert bits_equal(h1.weight(l), h2.weight(l))
+        assert bits_equal(h1.bias(l), h2.bias(l))
+    assert bits_equal(h1.dx(), h2.dx())
     h1.close(); h2.close()
 
 
@@ -87,13 +91,16 @@ def test_graph_replay_matches_eager_over_several_steps():
     nf, B, R = CONFIGS["C1_tiny"]
     hg, _ = build(nf, B, R, seed=11, flags=0)
     he, _ = build(nf, B, R, seed=11, flags=capi.FLAG_NO_GRAPH)
+    lr = 1e-4  # small enough that six sum-reduced steps stay finite
     for step in range(6):
-        hg.step(LR)
-        he.step(LR)
+        hg.step(lr)
+        he.step(lr)
         hg.sync(); he.sync()
         for l in range(len(nf) - 1):
-            assert np.array_equal(hg.weight(l), he.weight(l)), (step, l)
-        assert np.array_equal(hg.dx(), he.dx()), step
+            w = hg.weight(l)
+            assert np.all(np.isfinite(w))
+            assert bits_equal(w, he.weight(l)), (step, l)
+        assert bits_equal(hg.dx(), he.dx()), step
     hg.close(); he.close()
 
 
@@ -127,11 +134,23 @@ def test_timing_slots_are_filled():
 
 
 def test_benchmark_config_2_full_size():
-    """Benchmark config 2 (8 x 1024, batch 1024 x 4 replicas) at full size against the oracle."""
+    """Benchmark config 2 (8 x 1024, batch 1024 x 4 replicas) at full size against the oracle.
+    The forward pass is compared directly.  With 29 M ReLU inputs a handful of them lie within
+    rounding distance of zero, where the mask [A > 0] of an fp32 and a float64-accumulating
+    forward pass may legitimately differ and flip whole gradient entries; the backward pass is
+    therefore compared with the oracle evaluated on the device's own activations."""
     nf, B, R = [1024] * 9, 1024, 4
+    L = len(nf) - 1
     h, (X, Ws, bs, dY) = build(nf, B, R, seed=42)
     ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR)
     h.step(LR)
     h.sync()
-    compare_step(h, ref, nf, R)
+    acts = [h.activation(l) for l in range(L + 1)]
+    flips = 0
+    for l in range(L + 1):
+        assert rel_err(acts[l], ref.acts[l]) <= FP32_TOL, f"activation {l}"
+        flips += int(np.count_nonzero((acts[l] > 0) != (ref.acts[l] > 0)))
+    assert flips < 100, f"{flips} mask disagreements: more than rounding explains"
+    ref_b = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR, given_acts=acts)
+    compare_step(h, ref_b, nf, R, forward=False)
     h.close()
