@@ -186,11 +186,8 @@ int op_wgrad(mi_mlp* h, int l, hipStream_t s, bool with_bias) {
   hipError_t e;
   if (h->dtype == MI_F32) {
     e = mi::sgemm_tn(h->R, h->nf[l + 1], h->nf[l], h->B, (const float*)dz_of_layer(h, l), h->nf[l + 1],
-                     (const float*)h->acts[l], h->nf[l], const_cast<float*>(g0), h->nf[l], (long long)h->stride, s,
-                     g_variant[2]);
-    if (e == hipSuccess && with_bias)
-      e = mi::colsum_f32(h->R, h->nf[l + 1], h->B, (const float*)dz_of_layer(h, l), h->nf[l + 1],
-                         h->grads + h->boff[l], (long long)h->stride, s);
+                     (const float*)h->acts[l], h->nf[l], const_cast<float*>(g0), h->nf[l], (long long)h->stride,
+                     with_bias ? h->grads + h->boff[l] : nullptr, (long long)h->stride, s, g_variant[2]);
   } else {
     return fail(MI_ERR_UNSUPPORTED, "bf16 weight gradient is not implemented in this build");
   }
@@ -424,8 +421,8 @@ int mi_sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const float
   if (int rc = check_gemm(M, N, K, A, lda, M, B, ldb, N, C, ldc)) return rc;
   MI_REQUIRE(R == 1 || strideC >= (long long)(M > 0 ? (size_t)(M - 1) * ldc + N : 0), "strideC overlaps replicas");
   MI_REQUIRE(!colsum || R == 1 || stride_colsum >= M, "stride_colsum overlaps replicas");
-  hipError_t e = mi::sgemm_tn(R, M, N, K, A, lda, B, ldb, C, ldc, strideC, as_stream(stream), g_variant[2]);
-  if (e == hipSuccess && colsum) e = mi::colsum_f32(R, M, K, A, lda, colsum, stride_colsum, as_stream(stream));
+  hipError_t e = mi::sgemm_tn(R, M, N, K, A, lda, B, ldb, C, ldc, strideC, colsum, stride_colsum, as_stream(stream),
+                              g_variant[2]);
   if (e != hipSuccess) return hip_fail(e, "mi_sgemm_tn launch");
   return MI_OK;
 }

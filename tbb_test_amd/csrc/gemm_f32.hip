@@ -50,6 +50,9 @@ struct GemmArgs {
   int relu;           // EPI_BIAS_RELU
   const float* mask;  // EPI_MASK: [M x N], result zeroed where mask <= 0
   int ldmask;
+  // fused column sums of the A operand (TN only): colsum[z*batchColsum + m] = sum_k A[k][m]
+  float* colsum;
+  long long batchColsum;
   // tile rasterisation
   int tiles_m, tiles_n;
 };
@@ -67,6 +70,14 @@ __device__ __forceinline__ void tile_of_block(const GemmArgs& p, int& tm, int& t
   }
   tm = id / p.tiles_n;
   tn = id - tm * p.tiles_n;
+}
+
+// Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does not wait for
+// global loads still in flight, so prefetches may cross it.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 template <int ROWS, int BK, bool KMAJOR>
@@ -148,8 +159,25 @@ __device__ __forceinline__ void load_frag(float (&frag)[TB][4], const float* lds
   }
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, int EPI>
+// COLSUM (weight gradient only, A stored [k][m]): the workgroups of tile column 0 also add up the
+// columns of their A tile while it sits in LDS -- thread j < BM owns column j and walks k in
+// order, so the sum is deterministic -- and write the bias gradient at the end.  The extra LDS
+// reads and adds run in the shadow of the MFMAs.
+//
+// STAGES selects the software pipeline:
+//   2  two LDS buffers; loads of step t+1 are issued at the top of step t, written to LDS at its
+//      end, one barrier per step at the step boundary.
+//   3  three LDS buffers; the tile of step t+1 (loaded during step t-1) is written to LDS at the
+//      top of step t, the loads of step t+2 are issued right after, and the one barrier per step
+//      sits in the middle of the step, where it only has to absorb the skew between wavefronts.
+//      Step boundaries carry no synchronisation at all, and the operand fragments of the next
+//      8-wide K chunk are always fetched from LDS while the current chunk is multiplied.
+template <int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM = false,
+          int STAGES = 2>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
+  static_assert(STAGES == 2 || STAGES == 3, "two or three LDS buffers");
+  static_assert(STAGES == 2 || (BK / 8) % 2 == 0, "the 3-stage loop alternates two fragment sets per chunk");
+  static_assert(!COLSUM || (!A_KMAJOR && BM <= WM * WN * 64), "fused column sums need A stored [k][m]");
   constexpr int NT = WM * WN * 64;
   constexpr int WTM = BM / WM, WTN = BN / WN;  // wavefront sub-tile
   constexpr int TM = WTM / 32, TN = WTN / 32;  // 32x32 blocks per wavefront
@@ -163,9 +191,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
   constexpr int NVA = TA::kVecs / NT, NVB = TB::kVecs / NT;
 
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  // LDS layout: [A buffer 0][A buffer 1][B buffer 0][B buffer 1]
+  // LDS layout: [A buffers 0..STAGES-1][B buffers 0..STAGES-1]
   auto As = [&](int buf) { return smem + buf * TA::kFloats; };
-  auto Bs = [&](int buf) { return smem + 2 * TA::kFloats + buf * TB::kFloats; };
+  auto Bs = [&](int buf) { return smem + STAGES * TA::kFloats + buf * TB::kFloats; };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -193,93 +221,164 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
+  const bool do_colsum = COLSUM && p.colsum != nullptr && tile_n == 0 && tid < BM;
+  float csum = 0.0f;
+
   f32x4 ra[NVA], rb[NVB];
+  const int nk = p.K / BK;
+  auto mfma_chunk = [&](const float (&fa)[TM][4], const float (&fb)[TN][4]) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q], acc[i][j], 0, 0, 0);
+  };
+  auto colsum_step = [&](const float* a_tile) {
+    const float* col = a_tile + tid;
+#pragma unroll
+    for (int k = 0; k < BK; ++k) csum += col[k * TA::kStride];
+  };
+
   load_tile<BM, BK, A_KMAJOR, NT, NVA>(ra, a_ptr, p.lda, tid);
   load_tile<BN, BK, B_KMAJOR, NT, NVB>(rb, b_ptr, p.ldb, tid);
   store_tile<BM, BK, A_KMAJOR, NT, NVA>(As(0), ra, tid);
   store_tile<BN, BK, B_KMAJOR, NT, NVB>(Bs(0), rb, tid);
-  __syncthreads();
 
-  const int nk = p.K / BK;
-  for (int t = 0; t < nk; ++t) {
-    const int cur = t & 1;
-    if (t + 1 < nk) {
+  if constexpr (STAGES == 2) {
+    __syncthreads();
+    for (int t = 0; t < nk; ++t) {
+      const int cur = t & 1;
+      if (t + 1 < nk) {
+        a_ptr += a_step;
+        b_ptr += b_step;
+        load_tile<BM, BK, A_KMAJOR, NT, NVA>(ra, a_ptr, p.lda, tid);
+        load_tile<BN, BK, B_KMAJOR, NT, NVB>(rb, b_ptr, p.ldb, tid);
+      }
+#pragma unroll
+      for (int kk = 0; kk < BK / 8; ++kk) {
+        float fa[TM][4], fb[TN][4];
+        load_frag<BM, BK, A_KMAJOR, TM>(fa, As(cur), wm0, kk, lane);
+        load_frag<BN, BK, B_KMAJOR, TN>(fb, Bs(cur), wn0, kk, lane);
+        mfma_chunk(fa, fb);
+      }
+      if (COLSUM && do_colsum) colsum_step(As(cur));
+      if (t + 1 < nk) {
+        store_tile<BM, BK, A_KMAJOR, NT, NVA>(As(cur ^ 1), ra, tid);
+        store_tile<BN, BK, B_KMAJOR, NT, NVB>(Bs(cur ^ 1), rb, tid);
+      }
+      __syncthreads();
+    }
+  } else {
+    constexpr int CH = BK / 8;  // 8-wide K chunks per step
+    if (nk > 1) {
       a_ptr += a_step;
       b_ptr += b_step;
       load_tile<BM, BK, A_KMAJOR, NT, NVA>(ra, a_ptr, p.lda, tid);
       load_tile<BN, BK, B_KMAJOR, NT, NVB>(rb, b_ptr, p.ldb, tid);
     }
-
+    lds_barrier();
+    float fa[2][TM][4], fb[2][TN][4];
+    load_frag<BM, BK, A_KMAJOR, TM>(fa[0], As(0), wm0, 0, lane);
+    load_frag<BN, BK, B_KMAJOR, TN>(fb[0], Bs(0), wn0, 0, lane);
+    int cur = 0;
+    for (int t = 0; t < nk; ++t) {
+      const int nxt = cur == 2 ? 0 : cur + 1;
 #pragma unroll
-    for (int kk = 0; kk < BK / 8; ++kk) {
-      float fa[TM][4], fb[TN][4];
-      load_frag<BM, BK, A_KMAJOR, TM>(fa, As(cur), wm0, kk, lane);
-      load_frag<BN, BK, B_KMAJOR, TN>(fb, Bs(cur), wn0, kk, lane);
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q], acc[i][j], 0, 0, 0);
+      for (int kk = 0; kk < CH; ++kk) {
+        const int fc = kk & 1, fn = fc ^ 1;
+        // fragments of the next chunk: same buffer, or chunk 0 of the next step's buffer (made
+        // visible by this step's barrier, which lies before the last chunk)
+        if (kk + 1 < CH) {
+          load_frag<BM, BK, A_KMAJOR, TM>(fa[fn], As(cur), wm0, kk + 1, lane);
+          load_frag<BN, BK, B_KMAJOR, TN>(fb[fn], Bs(cur), wn0, kk + 1, lane);
+        } else if (t + 1 < nk) {
+          load_frag<BM, BK, A_KMAJOR, TM>(fa[fn], As(nxt), wm0, 0, lane);
+          load_frag<BN, BK, B_KMAJOR, TN>(fb[fn], Bs(nxt), wn0, 0, lane);
+        }
+        if (kk == 0) {
+          if (t + 1 < nk) {  // tile t+1 was loaded a whole step ago
+            store_tile<BM, BK, A_KMAJOR, NT, NVA>(As(nxt), ra, tid);
+            store_tile<BN, BK, B_KMAJOR, NT, NVB>(Bs(nxt), rb, tid);
+          }
+          if (t + 2 < nk) {
+            a_ptr += a_step;
+            b_ptr += b_step;
+            load_tile<BM, BK, A_KMAJOR, NT, NVA>(ra, a_ptr, p.lda, tid);
+            load_tile<BN, BK, B_KMAJOR, NT, NVB>(rb, b_ptr, p.ldb, tid);
+          }
+        }
+        mfma_chunk(fa[fc], fb[fc]);
+        if (kk == CH - 2) lds_barrier();
+        if (kk == CH - 1 && COLSUM && do_colsum) colsum_step(As(cur));
+      }
+      cur = nxt;
     }
-
-    if (t + 1 < nk) {
-      store_tile<BM, BK, A_KMAJOR, NT, NVA>(As(cur ^ 1), ra, tid);
-      store_tile<BN, BK, B_KMAJOR, NT, NVB>(Bs(cur ^ 1), rb, tid);
-    }
-    __syncthreads();
   }
 
+  if (COLSUM && do_colsum) p.colsum[(size_t)blockIdx.z * p.batchColsum + m0 + tid] = csum;
+
   // ---- epilogue: registers -> global, fused bias/ReLU or ReLU mask --------------------------
+  // Column of (block j, value e) held by this lane: K-major B keeps the blocks side by side,
+  // N-major B interleaves them so that the lane owns TN consecutive columns (one vector store).
   const int l32 = lane & 31, hi = lane >> 5;
+  const int col0 = n0 + wn0 + (B_KMAJOR ? l32 : TN * l32);
+  constexpr int CSTEP = B_KMAJOR ? 32 : 1;
+  const float* __restrict__ mask = p.mask;
+
+  float bias_v[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) bias_v[j] = (EPI == EPI_BIAS_RELU && p.bias) ? p.bias[col0 + j * CSTEP] : 0.0f;
+
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
+    // rows of accumulator registers r = 0..15 of block row i
+    auto row_of = [&](int r) {
+      const int rb32 = 8 * (r >> 2) + 4 * hi + (r & 3);
+      return m0 + wm0 + (A_KMAJOR ? i * 32 + rb32 : TM * rb32 + i);
+    };
+    // all mask reads of this block row first, so that they are in flight together
+    float mk[16][TN];
+    if (EPI == EPI_MASK) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float* mrow = mask + (size_t)row_of(r) * p.ldmask + col0;
+        if (!B_KMAJOR && TN == 4) {
+          const f32x4 t = *reinterpret_cast<const f32x4*>(mrow);
+          mk[r][0] = t[0]; mk[r][1 % TN] = t[1]; mk[r][2 % TN] = t[2]; mk[r][3 % TN] = t[3];
+        } else if (!B_KMAJOR && TN == 2) {
+          const f32x2 t = *reinterpret_cast<const f32x2*>(mrow);
+          mk[r][0] = t[0]; mk[r][1 % TN] = t[1];
+        } else {
+#pragma unroll
+          for (int j = 0; j < TN; ++j) mk[r][j] = mrow[j * CSTEP];
+        }
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int rb32 = 8 * (r >> 2) + 4 * hi + (r & 3);  // row inside the 32x32 block
-      const int row = m0 + wm0 + (A_KMAJOR ? i * 32 + rb32 : TM * rb32 + i);
-      float* crow = C + (size_t)row * p.ldc;
-      if (B_KMAJOR) {
+      float* crow = C + (size_t)row_of(r) * p.ldc + col0;
+      float v[TN];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          const int col = n0 + wn0 + j * 32 + l32;
-          float v = acc[i][j][r];
-          if (EPI == EPI_BIAS_RELU) {
-            if (p.bias) v += p.bias[col];
-            if (p.relu) v = v > 0.0f ? v : 0.0f;
-          } else if (EPI == EPI_MASK) {
-            if (!(p.mask[(size_t)row * p.ldmask + col] > 0.0f)) v = 0.0f;
-          }
-          crow[col] = v;
-        }
-      } else {
-        // interleaved columns: this lane owns TN consecutive columns -> one vector store
-        const int col = n0 + wn0 + TN * l32;
-        float v[TN];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
+      for (int j = 0; j < TN; ++j) {
+        v[j] = acc[i][j][r];
         if (EPI == EPI_BIAS_RELU) {
-#pragma unroll
-          for (int j = 0; j < TN; ++j) {
-            if (p.bias) v[j] += p.bias[col + j];
-            if (p.relu) v[j] = v[j] > 0.0f ? v[j] : 0.0f;
-          }
+          v[j] += bias_v[j];
+          if (p.relu) v[j] = v[j] > 0.0f ? v[j] : 0.0f;
         } else if (EPI == EPI_MASK) {
-          const float* mrow = p.mask + (size_t)row * p.ldmask + col;
+          if (!(mk[r][j] > 0.0f)) v[j] = 0.0f;
+        }
+      }
+      if (!B_KMAJOR && TN == 4) {
+        const f32x4 o = {v[0], v[1 % TN], v[2 % TN], v[3 % TN]};
+        *reinterpret_cast<f32x4*>(crow) = o;
+      } else if (!B_KMAJOR && TN == 2) {
+        const f32x2 o = {v[0], v[1 % TN]};
+        *reinterpret_cast<f32x2*>(crow) = o;
+      } else {
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            if (!(mrow[j] > 0.0f)) v[j] = 0.0f;
-        }
-        if (TN == 4) {
-          f32x4 o = {v[0], v[1 % TN], v[2 % TN], v[3 % TN]};
-          *reinterpret_cast<f32x4*>(crow + col) = o;
-        } else if (TN == 2) {
-          f32x2 o = {v[0], v[1 % TN]};
-          *reinterpret_cast<f32x2*>(crow + col) = o;
-        } else {
-          crow[col] = v[0];
-        }
+        for (int j = 0; j < TN; ++j) crow[j * CSTEP] = v[j];
       }
     }
   }
@@ -351,12 +450,12 @@ __global__ __launch_bounds__(256) void gemm_f32_generic(GemmArgs p) {
 
 // ---- launch ------------------------------------------------------------------------------------
 
-template <int BM, int BN, int BK, int WM, int WN, bool AK, bool BKM, int EPI>
+template <int BM, int BN, int BK, int WM, int WN, bool AK, bool BKM, int EPI, bool COLSUM, int STAGES = 2>
 static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
   using TA = TileShape<BM, BK, AK>;
   using TB = TileShape<BN, BK, BKM>;
-  constexpr size_t lds_bytes = 2 * (TA::kFloats + TB::kFloats) * sizeof(float);
-  auto kern = gemm_f32_mfma<BM, BN, BK, WM, WN, AK, BKM, EPI>;
+  constexpr size_t lds_bytes = STAGES * (TA::kFloats + TB::kFloats) * sizeof(float);
+  auto kern = gemm_f32_mfma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES>;
   static bool attr_set = false;  // opt in to more than 64 KiB of dynamic LDS once per kernel
   if (lds_bytes > 64 * 1024 && !attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -381,29 +480,48 @@ static hipError_t launch_generic(GemmArgs& p, int batch, hipStream_t s) {
 static inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 
 // Picks a tile configuration.  `variant` (0 = automatic) lets the tuning harness force one.
-template <bool AK, bool BKM, int EPI>
-static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant) {
+// `fused_colsum` reports whether the chosen kernel also produced p.colsum.
+template <bool AK, bool BKM, int EPI, bool COLSUM = false>
+static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, bool* fused_colsum = nullptr) {
+  if (fused_colsum) *fused_colsum = false;
   if (p.M <= 0 || p.N <= 0 || batch <= 0) return hipSuccess;
   const bool vec_ok = aligned16(p.A) && aligned16(p.B) && aligned16(p.C) && p.lda % 4 == 0 &&
                       p.ldb % 4 == 0 && p.ldc % 4 == 0 && p.batchA % 4 == 0 && p.batchB % 4 == 0 &&
                       p.batchC % 4 == 0 && p.K > 0;
   auto fits = [&](int bm, int bn, int bk) { return vec_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0; };
   if (variant == 0) {
-    // automatic choice: the largest tile that still yields at least one workgroup per CU
+    // Automatic choice.  One 128 x 128 tile per CU (or more) keeps the chip busy with the
+    // 8-wavefront, 3-stage kernel; the input-gradient GEMM gains a little from 128 x 64 tiles when
+    // that only just covers the CUs; small problems fall back to 64 x 64 tiles to get enough
+    // workgroups.
     const long long tiles128 = (long long)(p.M / 128) * (p.N / 128) * batch;
-    if (fits(256, 128, 32) && (long long)(p.M / 256) * (p.N / 128) * batch >= 512) variant = 3;
-    else if (fits(128, 128, 32) && tiles128 >= 128) variant = 1;
-    else if (fits(64, 64, 32)) variant = 4;
-    else variant = -1;
+    if (fits(128, 128, 32) && tiles128 >= 192) {
+      variant = (AK && !BKM && tiles128 <= 256 && fits(128, 64, 32)) ? 11 : 8;
+    } else if (fits(128, 64, 32) && tiles128 * 2 >= 192) {
+      variant = 11;
+    } else if (fits(64, 64, 16)) {
+      variant = 16;
+    } else {
+      variant = -1;
+    }
   }
   switch (variant) {
-    case 1: if (fits(128, 128, 32)) return launch_mfma<128, 128, 32, 2, 2, AK, BKM, EPI>(p, batch, s); break;
-    case 2: if (fits(128, 128, 32)) return launch_mfma<128, 128, 32, 2, 4, AK, BKM, EPI>(p, batch, s); break;
-    case 3: if (fits(256, 128, 32)) return launch_mfma<256, 128, 32, 2, 2, AK, BKM, EPI>(p, batch, s); break;
-    case 4: if (fits(64, 64, 32)) return launch_mfma<64, 64, 32, 2, 2, AK, BKM, EPI>(p, batch, s); break;
-    case 5: if (fits(128, 128, 16)) return launch_mfma<128, 128, 16, 2, 2, AK, BKM, EPI>(p, batch, s); break;
-    case 6: if (fits(256, 128, 16)) return launch_mfma<256, 128, 16, 4, 2, AK, BKM, EPI>(p, batch, s); break;
-    case 7: if (fits(128, 64, 32)) return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI>(p, batch, s); break;
+    case 1: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
+    case 2: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
+    case 3: if (fits(256, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<256, 128, 32, 2, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
+    case 4: if (fits(64, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<64, 64, 32, 2, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
+    case 5: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 16, 2, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
+    case 6: if (fits(256, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<256, 128, 16, 4, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
+    case 7: if (fits(128, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
+    case 8: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 9: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 10: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 11: if (fits(128, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 12: if (fits(128, 64, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 16, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 13: if (fits(64, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<64, 128, 16, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 14: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 16, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 15: if (fits(128, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI, COLSUM, 2>(p, batch, s); } break;
+    case 16: if (fits(64, 64, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<64, 64, 16, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     default: break;
   }
   return launch_generic<AK, BKM, EPI>(p, batch, s);
@@ -427,13 +545,20 @@ hipError_t sgemm_nn(int M, int N, int K, const float* A, int lda, const float* B
 }
 
 hipError_t sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
-                    float* C, int ldc, long long strideC, hipStream_t s, int variant) {
+                    float* C, int ldc, long long strideC, float* colsum, long long stride_colsum,
+                    hipStream_t s, int variant) {
   GemmArgs p{};
   p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.batchA = (long long)K * lda;  // replica r reads rows [r*K, (r+1)*K) of both operands
   p.batchB = (long long)K * ldb;
   p.batchC = strideC;
-  return dispatch<false, false, EPI_NONE>(p, R, s, variant);
+  if (!colsum) return dispatch<false, false, EPI_NONE>(p, R, s, variant);
+  p.colsum = colsum;
+  p.batchColsum = stride_colsum;
+  bool fused = false;
+  hipError_t e = dispatch<false, false, EPI_NONE, true>(p, R, s, variant, &fused);
+  if (e != hipSuccess || fused) return e;
+  return colsum_f32(R, M, K, A, lda, colsum, stride_colsum, s);  // any-shape path: separate kernel
 }
 
 }  // namespace mi

@@ -15,8 +15,10 @@ hipError_t sgemm_nt(int M, int N, int K, const float* A, int lda, const float* B
                     int ldc, const float* bias, int relu, hipStream_t s, int variant);
 hipError_t sgemm_nn(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
                     int ldc, const float* mask, int ldmask, hipStream_t s, int variant);
+// colsum (may be null): colsum[r*stride_colsum + m] = sum over replica r's K rows of A[.][m]
 hipError_t sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
-                    float* C, int ldc, long long strideC, hipStream_t s, int variant);
+                    float* C, int ldc, long long strideC, float* colsum, long long stride_colsum,
+                    hipStream_t s, int variant);
 
 // out[r*stride_out + j] = sum_{i in [r*K, (r+1)*K)} A[i*lda + j], j in [0, M)
 hipError_t colsum_f32(int R, int M, int K, const float* A, int lda, float* out, long long stride_out,
