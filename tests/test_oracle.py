@@ -1,0 +1,323 @@
+"""Pins the CPU oracle (oracle/) before anything is compared with it.  No GPU.
+
+What fixes each oracle function, besides its own formula:
+  GEMMs            numpy float64 matmul (a library routine), identity / one-hot / sign special cases
+  whole step       finite differences of the scalar <dY, output> in float64 (catches a dropped term,
+                   a transposed operand, a wrong mask), R-replica split == one big batch
+  reduce + SGD     the reference's closed-form start-up check (mlp_omp.cc:325-373), R = 1 == plain
+                   SGD, single-rounding of the fused multiply-add
+  partition        fixture sweep produced by the compiled reference Partition.cc, the compiled
+                   reference itself where built, spot values, tiling invariants
+  ring info        the reference's two ring tables (mlp_bench_common.cc:13-14) and ring invariants
+  seeded inputs    committed first-values fixture (pins the generator against drift only: the
+                   reference's MKL Niederreiter stream is not reproducible outside MKL)
+"""
+import ctypes
+import gzip
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle import partition as P
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+
+
+def rel(a, b):
+    return float(np.abs(np.asarray(a, np.float64) - b).max() / max(np.abs(b).max(), 1e-300))
+
+
+# ---- GEMMs -------------------------------------------------------------------------------------
+
+SHAPES = [(1, 1, 1), (3, 5, 7), (64, 48, 96), (129, 65, 33), (17, 1, 300)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_forward_matches_numpy_float64(M, N, K):
+    rng = np.random.default_rng(M * 1000 + N * 10 + K)
+    X = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    W = rng.uniform(-1, 1, (N, K)).astype(np.float32)
+    b = rng.uniform(-1, 1, N).astype(np.float32)
+    want = X.astype(np.float64) @ W.astype(np.float64).T + b
+    assert rel(oracle.fc_forward(X, W, b, False), want) < 1e-6
+    assert rel(oracle.fc_forward(X, W, None, False), want - b) < 1e-6
+    assert rel(oracle.fc_forward(X, W, b, True), np.maximum(want, 0)) < 1e-6
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_wgrad_and_dgrad_match_numpy_float64(M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    dZ = rng.standard_normal((K, M)).astype(np.float32)
+    A = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    dW, db = oracle.fc_wgrad(dZ, A)
+    assert rel(dW, dZ.astype(np.float64).T @ A.astype(np.float64)) < 1e-6
+    assert rel(db, dZ.astype(np.float64).sum(0)) < 1e-6
+    g = rng.standard_normal((M, K)).astype(np.float32)
+    W = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    act = np.maximum(rng.uniform(-1, 1, (M, N)), 0).astype(np.float32)
+    want = g.astype(np.float64) @ W.astype(np.float64)
+    assert rel(oracle.fc_dgrad(g, W), want) < 1e-6
+    assert rel(oracle.fc_dgrad(g, W, act), want * (act > 0)) < 1e-6
+
+
+def test_gemm_special_cases():
+    n = 16
+    rng = np.random.default_rng(0)
+    X = rng.uniform(-1, 1, (8, n)).astype(np.float32)
+    eye = np.eye(n, dtype=np.float32)
+    assert np.array_equal(oracle.fc_forward(X, eye), X)                      # identity weight
+    assert np.array_equal(oracle.fc_forward(np.abs(X), -eye, None, True), 0 * X)  # ReLU clamps negatives
+    assert np.array_equal(oracle.fc_forward(np.abs(X), eye, None, True), np.abs(X))  # and passes positives
+    W = rng.uniform(-1, 1, (n, 5)).astype(np.float32)
+    onehot = np.zeros((3, n), np.float32)
+    onehot[[0, 1, 2], [4, 9, 2]] = 1
+    assert np.array_equal(oracle.fc_dgrad(onehot, W), W[[4, 9, 2]])          # one-hot rows pick rows of W
+    # transposition check: a non-square, asymmetric case where X @ W (wrong) is not even defined
+    A = np.arange(6, dtype=np.float32).reshape(2, 3)
+    Wt = np.array([[1, 0, 0], [0, 2, 0], [0, 0, 3], [1, 1, 1]], np.float32)
+    assert np.array_equal(oracle.fc_forward(A, Wt), np.array([[0, 2, 6, 3], [3, 8, 15, 12]], np.float32))
+
+
+# ---- whole step: finite differences ---------------------------------------------------------------
+
+def _forward64(X, Ws, bs, relu_last):
+    A = X.astype(np.float64)
+    L = len(Ws)
+    for l in range(L):
+        Z = A @ Ws[l].T + bs[l]
+        A = np.maximum(Z, 0) if (l < L - 1 or relu_last) else Z
+    return A
+
+
+@pytest.mark.parametrize("relu_last", [False, True])
+def test_step_gradients_match_finite_differences(relu_last):
+    """With S(W, b, X) = <dY, output>, the step's sum over replicas of dW / db and its dX must be
+    the derivatives of S.  Central differences in float64 on a tiny model."""
+    nf, B, R = [5, 4, 6, 3], 3, 2
+    rng = np.random.default_rng(11)
+    MB = B * R
+    X = rng.uniform(-1, 1, (MB, nf[0])).astype(np.float32)
+    dY = rng.standard_normal((MB, nf[-1])).astype(np.float32)
+    Ws = [rng.uniform(-0.8, 0.8, (nf[l + 1], nf[l])).astype(np.float32) for l in range(3)]
+    bs = [rng.uniform(-0.3, 0.3, nf[l + 1]).astype(np.float32) for l in range(3)]
+    res = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, 0.0, relu_last=relu_last)
+
+    W64 = [w.astype(np.float64) for w in Ws]
+    b64 = [b.astype(np.float64) for b in bs]
+    S = lambda: float((dY.astype(np.float64) * _forward64(X, W64, b64, relu_last)).sum())
+    eps = 1e-6
+
+    def fd(arr, idx):
+        old = arr[idx]
+        arr[idx] = old + eps
+        up = S()
+        arr[idx] = old - eps
+        dn = S()
+        arr[idx] = old
+        return (up - dn) / (2 * eps)
+
+    for l in range(3):
+        gW = sum(res.dW[r][l].astype(np.float64) for r in range(R))
+        gb = sum(res.db[r][l].astype(np.float64) for r in range(R))
+        for idx in [(0, 0), (nf[l + 1] - 1, nf[l] - 1), (1, 2)]:
+            assert abs(fd(W64[l], idx) - gW[idx]) < 2e-4 * max(1.0, abs(gW[idx])), (l, idx)
+        for j in range(nf[l + 1]):
+            assert abs(fd(b64[l], j) - gb[j]) < 2e-4 * max(1.0, abs(gb[j])), (l, j)
+    X64 = X.astype(np.float64)
+
+    def S_x():
+        return float((dY.astype(np.float64) * _forward64(X64, W64, b64, relu_last)).sum())
+
+    for idx in [(0, 0), (MB - 1, nf[0] - 1), (2, 3)]:
+        old = X64[idx]
+        X64[idx] = old + eps
+        up = S_x()
+        X64[idx] = old - eps
+        dn = S_x()
+        X64[idx] = old
+        assert abs((up - dn) / (2 * eps) - res.dX[idx]) < 2e-4 * max(1.0, abs(res.dX[idx])), idx
+
+
+def test_step_replica_split_equals_one_big_batch():
+    """R replicas of batch B: activations and dX equal one replica of batch R*B, and the
+    per-replica gradients add up to the single-replica gradient."""
+    nf, B, R = [12, 9, 7], 4, 3
+    X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed=5)
+    a = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, 0.05)
+    b = oracle.mlp_step(nf, B * R, 1, X, dY, Ws, bs, 0.05)
+    assert np.array_equal(a.acts[-1], b.acts[-1]) and np.array_equal(a.dX, b.dX)
+    for l in range(2):
+        assert rel(sum(a.dW[r][l].astype(np.float64) for r in range(R)), b.dW[0][l].astype(np.float64)) < 1e-6
+        assert rel(a.W_new[l], b.W_new[l].astype(np.float64)) < 1e-6
+    # the update is W - lr * sum_r dW_r
+    want = Ws[0].astype(np.float64) - 0.05 * sum(a.dW[r][0].astype(np.float64) for r in range(R))
+    assert rel(a.W_new[0], want) < 1e-6
+
+
+# ---- reduce + SGD ----------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("R", [1, 2, 3, 4, 8])
+def test_reduce_sgd_reference_known_answer(R):
+    """mlp_omp.cc:325-373: G_r[i][j] = r + i + j, W[i][j] = i*j, lr = 1
+    =>  W' = i*j - ((i + j)*R + R*(R-1)/2), exact in fp32."""
+    rows, cols = 64, 80
+    i = np.arange(rows, dtype=np.float32)[:, None]
+    j = np.arange(cols, dtype=np.float32)[None, :]
+    W = (i * j).astype(np.float32)
+    G = np.stack([(r + i + j).astype(np.float32) for r in range(R)])
+    got = oracle.reduce_sgd(W.ravel(), G.reshape(R, -1), 1.0).reshape(rows, cols)
+    assert np.array_equal(got, (i * j - ((i + j) * R + R * (R - 1) / 2)).astype(np.float32))
+
+
+def test_reduce_sgd_is_single_rounding_fma_and_left_fold():
+    # lr * g = 1 + 2^-11 + 2^-24 exactly; rounded to fp32 first it becomes 1 + 2^-11 and the
+    # update of w = 1 + 2^-11 would be 0, while the single-rounding fma keeps the -2^-24
+    w = np.array([1.0 + 2.0 ** -11], np.float32)
+    g = np.array([[1.0 + 2.0 ** -12]], np.float32)
+    lr = np.float32(1.0 + 2.0 ** -12)
+    got = oracle.reduce_sgd(w, g, float(lr))
+    assert got[0] == np.float32(-(2.0 ** -24))
+    assert np.float32(np.float32(-lr * g[0, 0]) + w[0]) == 0.0
+    # left fold in replica order: (1e8 + 1) - 1e8 in fp32 is 0, not 1
+    G = np.array([[1e8], [1.0], [-1e8]], np.float32)
+    assert oracle.reduce_sgd(np.zeros(1, np.float32), G, -1.0)[0] == 0.0
+    G = np.array([[1e8], [-1e8], [1.0]], np.float32)
+    assert oracle.reduce_sgd(np.zeros(1, np.float32), G, -1.0)[0] == 1.0
+
+
+# ---- partition -------------------------------------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def golden():
+    with gzip.open(os.path.join(HERE, "golden", "partition_golden.json.gz"), "rt") as f:
+        return json.load(f)
+
+
+def test_partition_oracle_matches_reference_fixture(golden):
+    n = 0
+    for c in golden["partition_1d"]:
+        it = iter(c["ranges"])
+        for sid in range(c["ns"]):
+            for t in range(c["T"]):
+                assert list(P.partition_1d(c["work"], c["ns"], sid, c["T"], t)) == next(it), c
+                n += 1
+    for c in golden["partition_2d_intra"]:
+        for t, want in enumerate(c["blocks"]):
+            assert list(P.partition_2d_intra(c["m"], c["n"], c["ar"], bool(c["m_align"]), c["T"], t)) == want, (c, t)
+            n += 1
+    for c in golden["partition_2d"]:
+        it = iter(c["blocks"])
+        for sid in c["sids"]:
+            for t in range(c["T"]):
+                got = P.partition_2d(c["m"], c["n"], c["ar"], bool(c["m_align"]), c["ns"], sid, c["T"], t)
+                assert list(got) == next(it), (c["m"], c["n"], c["ar"], c["m_align"], c["ns"], sid, c["T"], t)
+                n += 1
+    assert n > 50000
+
+
+def test_partition_spot_values_from_a_reference_run():
+    assert P.partition_2d(4096, 1024, 4.0, False, 4, 0, 20, 0) == (0, 512, 0, 112)
+    assert P.partition_2d(4096, 1024, 4.0, False, 4, 0, 20, 19) == (512, 1024, 1008, 1024)
+    assert P.partition_2d(4096, 1024, 4.0, False, 4, 3, 20, 0) == (3072, 3584, 0, 112)
+    assert P.partition_2d_intra(1024, 1024, 0.5, True, 16, 0) == (0, 128, 0, 512)
+    assert P.partition_2d_intra(1024, 1024, 0.5, True, 16, 4) == (256, 384, 0, 512)
+    assert P.partition_2d_intra(1024, 1024, 0.5, True, 16, 15) == (896, 1024, 512, 1024)
+    assert P.partition_2d(512, 512, 4.0, False, 2, 1, 4, 2) == (256, 512, 256, 384)
+    assert P.partition_1d(1000, 2, 1, 4, 3) == (875, 1000)
+
+
+def test_partition_matches_compiled_reference_where_built():
+    path = os.path.join(ROOT, "oracle", "_ref", "libref_partition.so")
+    if not os.path.exists(path):
+        pytest.skip("oracle/_ref not built (needs the reference checkout)")
+    ref = ctypes.CDLL(path)
+    I = ctypes.c_int
+    ref.ref_get_2dpartition.argtypes = [I, I, ctypes.c_double, I, I, I, I, ctypes.POINTER(I)]
+    ref.ref_get_partition.argtypes = [I, I, I, I, ctypes.POINTER(I)]
+    out4, out2 = (I * 4)(), (I * 2)()
+    rng = np.random.default_rng(3)
+    for _ in range(3000):
+        ns = int(rng.choice([1, 2, 3, 4, 8]))
+        T = int(rng.integers(1, 33))
+        m, n = int(rng.integers(1, 5000)), int(rng.integers(1, 5000))
+        ar = float(rng.choice([4.0, 0.5, 1.0, 0.125, 32.0]))
+        ma = int(rng.integers(0, 2))
+        sid, t = int(rng.integers(0, ns)), int(rng.integers(0, T))
+        ref.ref_set_nsockets(ns)
+        ref.ref_get_2dpartition(m, n, ar, ma, sid, T, t, out4)
+        assert tuple(out4) == P.partition_2d(m, n, ar, bool(ma), ns, sid, T, t), (m, n, ar, ma, ns, sid, T, t)
+        ref.ref_get_partition(m, sid, T, t, out2)
+        assert tuple(out2) == P.partition_1d(m, ns, sid, T, t)
+
+
+@pytest.mark.parametrize("m,n,ar,m_align,ns,T", [(4096, 1024, 4.0, False, 4, 20), (1024, 1024, 0.5, True, 1, 16),
+                                                 (1000, 17, 0.5, True, 2, 10), (33, 129, 4.0, False, 8, 5),
+                                                 (8192, 1, 4.0, False, 2, 28)])
+def test_partition_blocks_tile_the_output_exactly_once(m, n, ar, m_align, ns, T):
+    cover = np.zeros((m, n), np.int32)
+    for sid in range(ns):
+        for t in range(T):
+            mb, me, nb, ne = P.partition_2d(m, n, ar, m_align, ns, sid, T, t)
+            assert 0 <= mb <= me <= m and 0 <= nb <= ne <= n
+            assert nb % 16 == 0 or nb == n
+            cover[mb:me, nb:ne] += 1
+    assert np.all(cover == 1)
+
+
+# ---- ring info -------------------------------------------------------------------------------------
+
+def test_ring_tables_and_invariants():
+    assert P.RINGS == ((0, 1, 2, 4, 7, 6, 5, 3), (0, 3, 5, 6, 7, 4, 2, 1))
+    assert P.RINGS[1][1:] == P.RINGS[0][:0:-1]  # the second ring is the first one walked backwards
+    for ns in (1, 2, 3, 4, 8):
+        for task in (0, 1, 2, 3):
+            nxt = {s: P.ring_info(s, task, ns)[2] for s in range(ns)}
+            prv = {s: P.ring_info(s, task, ns)[1] for s in range(ns)}
+            idx = sorted(P.ring_info(s, task, ns)[0] for s in range(ns))
+            assert idx == list(range(ns))
+            assert all(prv[nxt[s]] == s for s in range(ns))
+            s, seen = 0, set()
+            for _ in range(ns):  # following `next` visits every socket once
+                seen.add(s)
+                s = nxt[s]
+            assert seen == set(range(ns)) and s == 0
+    assert P.ring_info(4, 0, 8) == (3, 2, 7) and P.ring_info(4, 1, 8) == (5, 7, 2)
+    assert P.ring_info(1, 0, 4) == (1, 0, 2) and P.ring_info(1, 1, 4) == (1, 2, 0)
+
+
+# ---- seeded inputs ---------------------------------------------------------------------------------
+
+def test_numpy_generator_matches_committed_fixture():
+    with open(os.path.join(HERE, "golden", "rand_golden.json")) as f:
+        g = json.load(f)
+    for c in g["raw"]:
+        assert [int(v) for v in oracle.rand_raw(c["seed"], c["stream"], 0, 8)] == c["values"]
+    for c in g["uniform"]:
+        got = oracle.rand_uniform(c["seed"], c["stream"], 0, 16, c["low"], c["high"])
+        assert [float(v).hex() for v in got] == c["hex"]
+        assert np.all(got >= np.float32(c["low"])) and np.all(got <= np.float32(c["high"]))
+    for c in g["normal"]:
+        got = oracle.rand_normal(c["seed"], c["stream"], 0, 16)
+        want = np.array([float.fromhex(h) for h in c["hex"]], np.float32)
+        # libm vs numpy log/cos may differ in the last bit of the double before rounding to float
+        assert np.all(np.abs(got - want) <= np.spacing(np.abs(want)))
+    p = g["problem"]
+    X, Ws, bs, dY = oracle.make_problem(p["nf"], p["B"], p["R"], p["seed"])
+    assert [float(v).hex() for v in X[0]] == p["X_row0"]
+    assert [float(v).hex() for v in Ws[0][0]] == p["W0_row0"]
+    assert [float(v).hex() for v in Ws[1][0]] == p["W1_row0"]
+    assert all(not b.any() for b in bs)
+
+
+def test_generator_distributions():
+    u = oracle.rand_uniform(3, 0, 0, 200000, -1.0, 1.0)
+    assert abs(u.mean()) < 0.01 and abs(u.var() - 1 / 3) < 0.01 and u.min() >= -1 and u.max() < 1
+    z = oracle.rand_normal(3, 1000, 0, 200000)
+    assert abs(z.mean()) < 0.01 and abs(z.std() - 1) < 0.01 and np.all(np.isfinite(z))
+    a = np.sqrt(6.0 / (512 + 512))
+    _, Ws, _, _ = oracle.make_problem([512, 512], 4, 1, 9)
+    assert Ws[0].max() <= np.float32(a) and Ws[0].min() >= -np.float32(a) and abs(Ws[0].std() - a / np.sqrt(3)) < 1e-3
