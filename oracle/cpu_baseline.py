@@ -1,48 +1,123 @@
-"""CPU baseline leg of bench.py: times the CPU restatement of the reference path on this host.
+"""CPU baseline leg of bench.py: times the OpenMP restatement of the reference's mlp_omp
+(oracle/mlp_omp_port.c) on this host's cores.
 
-TEST / MEASUREMENT INFRASTRUCTURE ONLY.  The number it produces is a reported baseline, not a
-target: the reference itself (MKL + TBB) cannot be built in this image, so the timed code is this
-repository's own restatement ("kind": "port").
+TEST / MEASUREMENT INFRASTRUCTURE ONLY.  The number is a reported baseline, not a target.  The
+reference itself (MKL + TBB) cannot be built in this image, so the timed code is this repository's
+restatement ("kind": "port"): same thread layout, same 2-D work partition, same ring
+reduce-scatter / all-gather with fused SGD, one sequential SGEMM call per thread.  SGEMM is
+OpenBLAS as shipped inside scipy (single-threaded per call, like the reference uses MKL), or the
+built-in kernel of the port when that library cannot be found.
 """
+import ctypes
+import glob
 import os
-import time
+import subprocess
 
 import numpy as np
 
-import oracle
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_lib = None
+_vp, _ci = ctypes.c_void_p, ctypes.c_int
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        path = os.path.join(_HERE, "libmlp_omp_port.so")
+        if not os.path.exists(path):
+            subprocess.check_call(["make", "-C", _HERE, "libmlp_omp_port.so"], stdout=subprocess.DEVNULL)
+        l = ctypes.CDLL(path)
+        l.port_mlp_run.argtypes = [_ci, ctypes.POINTER(_ci), _ci, _ci, _ci, ctypes.c_float, _ci, _vp, _vp, _vp, _ci,
+                                   _ci, _ci, _vp, _vp, _vp, ctypes.POINTER(ctypes.c_double)]
+        l.port_mlp_run.restype = _ci
+        l.port_check_all_reduce.argtypes = [_ci, _ci, _ci, _ci]
+        l.port_check_all_reduce.restype = _ci
+        l.port_partition_2d.argtypes = [_ci, _ci, ctypes.c_double, _ci, _ci, _ci, _ci, _ci, ctypes.POINTER(_ci)]
+        l.port_partition_2d_intra.argtypes = [_ci, _ci, ctypes.c_double, _ci, _ci, _ci, ctypes.POINTER(_ci)]
+        l.port_ring_info.argtypes = [_ci, _ci, _ci, ctypes.POINTER(_ci)]
+        _lib = l
+    return _lib
+
+
+_blas = None
+
+
+def find_sgemm():
+    """(address of a cblas_sgemm-compatible function or None, description)."""
+    global _blas
+    if _blas is not None:
+        return _blas
+    _blas = (None, "built-in blocked SGEMM of the port")
+    try:
+        import scipy
+        pattern = os.path.join(os.path.dirname(os.path.dirname(scipy.__file__)), "scipy.libs", "libscipy_openblas*.so")
+        for path in sorted(glob.glob(pattern)):
+            blas = ctypes.CDLL(path)
+            if hasattr(blas, "scipy_cblas_sgemm"):
+                if hasattr(blas, "scipy_openblas_set_num_threads"):
+                    blas.scipy_openblas_set_num_threads(1)
+                addr = ctypes.cast(blas.scipy_cblas_sgemm, _vp).value
+                _blas = (addr, f"OpenBLAS cblas_sgemm ({os.path.basename(path)}), 1 thread per call")
+                _blas_keepalive.append(blas)
+                break
+    except Exception:
+        pass
+    return _blas
+
+
+_blas_keepalive = []
+
+
+def host_cores():
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    return max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
+
+
+def run_port(nf, B, R, T, lr, X, dY, W_flat, warmup, iters, restore=True, relu_last=False, use_blas=True):
+    """One call of the C port.  Returns (W_out flat, dX, times_ms[5])."""
+    L = len(nf) - 1
+    MB = B * R
+    X = np.ascontiguousarray(X, np.float32)
+    dY = np.ascontiguousarray(dY, np.float32)
+    W_flat = np.ascontiguousarray(W_flat, np.float32)
+    W_out = np.empty_like(W_flat)
+    dX = np.empty((MB, nf[0]), np.float32)
+    times = (ctypes.c_double * 5)()
+    arr = (_ci * len(nf))(*nf)
+    sgemm = find_sgemm()[0] if use_blas else None
+    rc = lib().port_mlp_run(L, arr, B, R, T, lr, int(relu_last), X.ctypes.data_as(_vp), dY.ctypes.data_as(_vp),
+                            W_flat.ctypes.data_as(_vp), warmup, iters, int(restore), sgemm,
+                            W_out.ctypes.data_as(_vp), dX.ctypes.data_as(_vp), times)
+    if rc != 0:
+        raise RuntimeError(f"port_mlp_run failed with {rc}")
+    return W_out, dX, list(times)
 
 
 def run(nf, B, R, lr, budget_s):
-    """Runs whole training steps of the given model on the host until about budget_s seconds of
-    CPU work are spent (at least one step), and returns the cpu_baseline object of the bench line.
-    If one full step does not fit the budget, the batch per replica is cut down (the work per step
-    is linear in it) and the sample says so."""
+    """The cpu_baseline object of the bench line: whole training steps of the given model, same
+    seeded inputs as the GPU run, for about budget_s seconds."""
+    import oracle
+
     L = len(nf) - 1
-    flop_full = 3 * 2.0 * R * B * sum(nf[l] * nf[l + 1] for l in range(L))
-    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
-    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-    # the double-accumulating oracle sustains roughly 2.5 GFLOP/s per core
-    est_step_s = flop_full / (2.5e9 * cores)
-    Bs = B
-    while Bs > 16 and est_step_s * Bs / B > budget_s:
-        Bs //= 2
-    X, Ws, bs, dY = oracle.make_problem(nf, Bs, R, seed=1)
-    flop = flop_full * Bs / B
-    steps, t0 = 0, time.perf_counter()
-    while True:
-        oracle.mlp_step(nf, Bs, R, X, dY, Ws, bs, lr)
-        steps += 1
-        spent = time.perf_counter() - t0
-        if spent + spent / steps > budget_s or steps >= 50:
-            break
-    ms = spent / steps * 1e3
+    cores = host_cores()
+    T = max(1, cores // R)
+    X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed=1)
+    W_flat = np.concatenate([np.concatenate([Ws[l].ravel(), bs[l].ravel()]) for l in range(L)])
+    flop = 3 * 2.0 * R * B * sum(nf[l] * nf[l + 1] for l in range(L))
+    _, _, t = run_port(nf, B, R, T, lr, X, dY, W_flat, 1, 1)          # warm caches, estimate the step time
+    iters = int(max(1, min(200, (budget_s - 2 * t[4] * 1e-3) / max(t[4] * 1e-3, 1e-6))))
+    _, _, t = run_port(nf, B, R, T, lr, X, dY, W_flat, 1, iters)
+    ms = t[4]
     return {
         "value": round(flop / (ms * 1e-3) / 1e12, 5),
         "unit": "TFLOP/s",
-        "cores": cores,
+        "cores": R * T,
         "kind": "port",
-        "ms_per_step": round(ms, 2),
-        "sample": f"{steps} full step(s) of the same model with batch {Bs} per replica x {R} replicas"
-                  f"{'' if Bs == B else f' (cut down from {B}; work per step is linear in the batch)'}, "
-                  "float64-accumulating OpenMP oracle (oracle/mlp_oracle.c)",
+        "ms_per_step": round(ms, 3),
+        "phase_ms_per_step": {"fwd": round(t[0], 3), "wgt_grad": round(t[1], 3), "bwd": round(t[2], 3),
+                              "wgt_update": round(t[3], 3)},
+        "sgemm": find_sgemm()[1],
+        "sample": f"{iters} full step(s) of the same workload (same model, batch and seeded inputs), "
+                  f"{R} replicas x {T} threads = {R * T} OpenMP threads on {cores} host cores, restatement of "
+                  "mlp_omp (oracle/mlp_omp_port.c)",
     }

@@ -1,0 +1,63 @@
+"""Pins the CPU baseline (oracle/mlp_omp_port.c, the OpenMP restatement of the reference's mlp_omp
+that bench.py times) against the float64-accumulating oracle, its ring all-reduce against the
+reference's closed-form start-up check (mlp_omp.cc:325-373), and its C restatement of the work
+partition against the fixture produced by the compiled reference.  No GPU."""
+import ctypes
+import gzip
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle import cpu_baseline as cb
+from oracle import partition as P
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+@pytest.mark.parametrize("ns,T", [(1, 1), (1, 3), (2, 2), (2, 5), (3, 2), (4, 2), (4, 4), (5, 3), (8, 1), (8, 2)])
+def test_ring_all_reduce_known_answer(ns, T):
+    assert cb.lib().port_check_all_reduce(64, 80, ns, T) == 0
+    assert cb.lib().port_check_all_reduce(33, 16, ns, T) == 0  # rows not a multiple of the socket count
+
+
+def test_port_partition_matches_reference_fixture():
+    with gzip.open(os.path.join(HERE, "golden", "partition_golden.json.gz"), "rt") as f:
+        golden = json.load(f)
+    out = (ctypes.c_int * 4)()
+    lib = cb.lib()
+    for c in golden["partition_2d"][::7]:
+        it = iter(c["blocks"])
+        for sid in c["sids"]:
+            for t in range(c["T"]):
+                lib.port_partition_2d(c["m"], c["n"], c["ar"], c["m_align"], c["ns"], sid, c["T"], t, out)
+                assert list(out) == next(it)
+    out3 = (ctypes.c_int * 3)()
+    for ns in (2, 4, 8):
+        for sid in range(ns):
+            for task in (0, 1):
+                lib.port_ring_info(ns, sid, task, out3)
+                assert tuple(out3) == P.ring_info(sid, task, ns)
+
+
+@pytest.mark.parametrize("nf,B,R,T,relu_last", [([96, 64, 80, 32], 24, 2, 2, False), ([64, 64, 64], 16, 4, 2, True),
+                                               ([100, 70, 33, 1], 10, 3, 1, False), ([48, 48], 8, 1, 4, False)])
+@pytest.mark.parametrize("use_blas", [True, False])
+def test_port_step_matches_oracle(nf, B, R, T, relu_last, use_blas):
+    L = len(nf) - 1
+    X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed=8)
+    rng = np.random.default_rng(2)
+    bs = [(0.1 * rng.standard_normal(b.shape)).astype(np.float32) for b in bs]
+    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, 0.01, relu_last=relu_last)
+    flat = np.concatenate([np.concatenate([Ws[l].ravel(), bs[l].ravel()]) for l in range(L)])
+    want = np.concatenate([np.concatenate([ref.W_new[l].ravel(), ref.b_new[l].ravel()]) for l in range(L)])
+    got, dX, times = cb.run_port(nf, B, R, T, 0.01, X, dY, flat, 0, 1, relu_last=relu_last, use_blas=use_blas)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    assert np.abs(dX - ref.dX).max() <= 1e-5 * max(np.abs(ref.dX).max(), 1e-30)
+    assert times[4] > 0
+    # restoring the weights before every step makes repeated steps idempotent
+    again, _, _ = cb.run_port(nf, B, R, T, 0.01, X, dY, flat, 1, 2, restore=True, relu_last=relu_last,
+                              use_blas=use_blas)
+    assert np.abs(again - want).max() <= 1e-5 * np.abs(want).max()
