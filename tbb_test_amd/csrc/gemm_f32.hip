@@ -160,9 +160,11 @@ __device__ __forceinline__ void load_frag(float (&frag)[TB][4], const float* lds
 }
 
 // COLSUM (weight gradient only, A stored [k][m]): the workgroups of tile column 0 also add up the
-// columns of their A tile while it sits in LDS -- thread j < BM owns column j and walks k in
-// order, so the sum is deterministic -- and write the bias gradient at the end.  The extra LDS
-// reads and adds run in the shadow of the MFMAs.
+// columns of their A tile while it sits in LDS.  Every thread takes part so that no wavefront
+// falls behind: thread t owns column t % BM and the k rows of slice t / BM of every K step; the
+// NT / BM partial sums of a column are combined through LDS in slice order at the end, so the
+// result does not depend on scheduling.  The extra LDS reads and adds run in the shadow of the
+// MFMAs.
 //
 // STAGES selects the software pipeline:
 //   2  two LDS buffers; loads of step t+1 are issued at the top of step t, written to LDS at its
@@ -172,12 +174,15 @@ __device__ __forceinline__ void load_frag(float (&frag)[TB][4], const float* lds
 //      sits in the middle of the step, where it only has to absorb the skew between wavefronts.
 //      Step boundaries carry no synchronisation at all, and the operand fragments of the next
 //      8-wide K chunk are always fetched from LDS while the current chunk is multiplied.
+//      PF (1 or 2) is the distance, in K steps, between issuing a tile's global loads and
+//      writing it to LDS; 2 covers an L2 miss without stalling the step that needs the data.
 template <int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM = false,
-          int STAGES = 2>
+          int STAGES = 2, int PF = 1>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
   static_assert(STAGES == 2 || STAGES == 3, "two or three LDS buffers");
   static_assert(STAGES == 2 || (BK / 8) % 2 == 0, "the 3-stage loop alternates two fragment sets per chunk");
-  static_assert(!COLSUM || (!A_KMAJOR && BM <= WM * WN * 64), "fused column sums need A stored [k][m]");
+  static_assert(!COLSUM || (!A_KMAJOR && (WM * WN * 64) % BM == 0 && BK % ((WM * WN * 64) / BM) == 0),
+                "fused column sums need A stored [k][m] and a whole number of k slices");
   constexpr int NT = WM * WN * 64;
   constexpr int WTM = BM / WM, WTN = BN / WN;  // wavefront sub-tile
   constexpr int TM = WTM / 32, TN = WTN / 32;  // 32x32 blocks per wavefront
@@ -221,7 +226,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  const bool do_colsum = COLSUM && p.colsum != nullptr && tile_n == 0 && tid < BM;
+  constexpr int CS_SLICES = COLSUM ? NT / BM : 1;  // k slices per step, one per group of BM threads
+  constexpr int CS_ROWS = BK / CS_SLICES;
+  const bool do_colsum = COLSUM && p.colsum != nullptr && tile_n == 0;  // uniform over the workgroup
   float csum = 0.0f;
 
   f32x4 ra[NVA], rb[NVB];
@@ -236,9 +243,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q], acc[i][j], 0, 0, 0);
   };
   auto colsum_step = [&](const float* a_tile) {
-    const float* col = a_tile + tid;
+    const float* col = a_tile + (tid / BM) * CS_ROWS * TA::kStride + (tid % BM);
 #pragma unroll
-    for (int k = 0; k < BK; ++k) csum += col[k * TA::kStride];
+    for (int k = 0; k < CS_ROWS; ++k) csum += col[k * TA::kStride];
   };
 
   load_tile<BM, BK, A_KMAJOR, NT, NVA>(ra, a_ptr, p.lda, tid);
@@ -272,18 +279,28 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
     }
   } else {
     constexpr int CH = BK / 8;  // 8-wide K chunks per step
-    if (nk > 1) {
+    // Global loads run PF steps ahead of their use.  With PF == 2 two register sets alternate:
+    // tiles with an odd index travel through (ra2, rb2), even ones through (ra, rb).
+    f32x4 ra2[PF == 2 ? NVA : 1], rb2[PF == 2 ? NVB : 1];
+    auto fetch = [&](auto& sa, auto& sb) {
       a_ptr += a_step;
       b_ptr += b_step;
-      load_tile<BM, BK, A_KMAJOR, NT, NVA>(ra, a_ptr, p.lda, tid);
-      load_tile<BN, BK, B_KMAJOR, NT, NVB>(rb, b_ptr, p.ldb, tid);
+      load_tile<BM, BK, A_KMAJOR, NT, NVA>(sa, a_ptr, p.lda, tid);
+      load_tile<BN, BK, B_KMAJOR, NT, NVB>(sb, b_ptr, p.ldb, tid);
+    };
+    if constexpr (PF == 2) {
+      if (nk > 1) fetch(ra2, rb2);
+      if (nk > 2) fetch(ra, rb);
+    } else {
+      if (nk > 1) fetch(ra, rb);
     }
     lds_barrier();
     float fa[2][TM][4], fb[2][TN][4];
     load_frag<BM, BK, A_KMAJOR, TM>(fa[0], As(0), wm0, 0, lane);
     load_frag<BN, BK, B_KMAJOR, TN>(fb[0], Bs(0), wn0, 0, lane);
     int cur = 0;
-    for (int t = 0; t < nk; ++t) {
+    // one K step; (sa, sb) hold tile t+1 on entry and receive tile t+1+PF
+    auto step = [&](int t, auto& sa, auto& sb) {
       const int nxt = cur == 2 ? 0 : cur + 1;
 #pragma unroll
       for (int kk = 0; kk < CH; ++kk) {
@@ -298,26 +315,39 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
           load_frag<BN, BK, B_KMAJOR, TN>(fb[fn], Bs(nxt), wn0, 0, lane);
         }
         if (kk == 0) {
-          if (t + 1 < nk) {  // tile t+1 was loaded a whole step ago
-            store_tile<BM, BK, A_KMAJOR, NT, NVA>(As(nxt), ra, tid);
-            store_tile<BN, BK, B_KMAJOR, NT, NVB>(Bs(nxt), rb, tid);
+          if (t + 1 < nk) {  // tile t+1 was requested PF whole steps ago
+            store_tile<BM, BK, A_KMAJOR, NT, NVA>(As(nxt), sa, tid);
+            store_tile<BN, BK, B_KMAJOR, NT, NVB>(Bs(nxt), sb, tid);
           }
-          if (t + 2 < nk) {
-            a_ptr += a_step;
-            b_ptr += b_step;
-            load_tile<BM, BK, A_KMAJOR, NT, NVA>(ra, a_ptr, p.lda, tid);
-            load_tile<BN, BK, B_KMAJOR, NT, NVB>(rb, b_ptr, p.ldb, tid);
-          }
+          if (t + 1 + PF < nk) fetch(sa, sb);
         }
         mfma_chunk(fa[fc], fb[fc]);
         if (kk == CH - 2) lds_barrier();
         if (kk == CH - 1 && COLSUM && do_colsum) colsum_step(As(cur));
       }
       cur = nxt;
+    };
+    if constexpr (PF == 2) {
+      for (int t = 0; t < nk; t += 2) {
+        step(t, ra2, rb2);
+        if (t + 1 < nk) step(t + 1, ra, rb);
+      }
+    } else {
+      for (int t = 0; t < nk; ++t) step(t, ra, rb);
     }
   }
 
-  if (COLSUM && do_colsum) p.colsum[(size_t)blockIdx.z * p.batchColsum + m0 + tid] = csum;
+  if (COLSUM && do_colsum) {
+    __syncthreads();  // every wavefront is done with the operand tiles: reuse LDS for the partials
+    smem[tid] = csum;
+    __syncthreads();
+    if (tid < BM) {
+      float total = smem[tid];
+#pragma unroll
+      for (int sl = 1; sl < CS_SLICES; ++sl) total += smem[sl * BM + tid];
+      p.colsum[(size_t)blockIdx.z * p.batchColsum + m0 + tid] = total;
+    }
+  }
 
   // ---- epilogue: registers -> global, fused bias/ReLU or ReLU mask --------------------------
   // Column of (block j, value e) held by this lane: K-major B keeps the blocks side by side,
@@ -450,12 +480,12 @@ __global__ __launch_bounds__(256) void gemm_f32_generic(GemmArgs p) {
 
 // ---- launch ------------------------------------------------------------------------------------
 
-template <int BM, int BN, int BK, int WM, int WN, bool AK, bool BKM, int EPI, bool COLSUM, int STAGES = 2>
+template <int BM, int BN, int BK, int WM, int WN, bool AK, bool BKM, int EPI, bool COLSUM, int STAGES = 2, int PF = 1>
 static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
   using TA = TileShape<BM, BK, AK>;
   using TB = TileShape<BN, BK, BKM>;
   constexpr size_t lds_bytes = STAGES * (TA::kFloats + TB::kFloats) * sizeof(float);
-  auto kern = gemm_f32_mfma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES>;
+  auto kern = gemm_f32_mfma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES, PF>;
   static bool attr_set = false;  // opt in to more than 64 KiB of dynamic LDS once per kernel
   if (lds_bytes > 64 * 1024 && !attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -491,12 +521,11 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
   auto fits = [&](int bm, int bn, int bk) { return vec_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0; };
   if (variant == 0) {
     // Automatic choice.  One 128 x 128 tile per CU (or more) keeps the chip busy with the
-    // 8-wavefront, 3-stage kernel; the input-gradient GEMM gains a little from 128 x 64 tiles when
-    // that only just covers the CUs; small problems fall back to 64 x 64 tiles to get enough
-    // workgroups.
+    // 8-wavefront, 3-stage kernel; smaller problems fall back to 128 x 64 and 64 x 64 tiles to
+    // get enough workgroups.
     const long long tiles128 = (long long)(p.M / 128) * (p.N / 128) * batch;
     if (fits(128, 128, 32) && tiles128 >= 192) {
-      variant = (AK && !BKM && tiles128 <= 256 && fits(128, 64, 32)) ? 11 : 8;
+      variant = 8;
     } else if (fits(128, 64, 32) && tiles128 * 2 >= 192) {
       variant = 11;
     } else if (fits(64, 64, 16)) {
@@ -522,6 +551,10 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
     case 14: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 16, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 15: if (fits(128, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI, COLSUM, 2>(p, batch, s); } break;
     case 16: if (fits(64, 64, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<64, 64, 16, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 17: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 3, 2>(p, batch, s); } break;
+    case 18: if (fits(128, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI, COLSUM, 3, 2>(p, batch, s); } break;
+    case 19: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3, 2>(p, batch, s); } break;
+    case 20: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 2, AK, BKM, EPI, COLSUM, 3, 2>(p, batch, s); } break;
     default: break;
   }
   return launch_generic<AK, BKM, EPI>(p, batch, s);

@@ -84,7 +84,7 @@ GEMM_SHAPES = [
     (64, 64, 32), (192, 64, 64),
     (1, 1, 1), (5, 3, 7), (100, 130, 50), (129, 127, 33), (257, 64, 1000), (64, 1, 64), (1, 300, 17),
 ]
-VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11]
+VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20]
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
