@@ -40,6 +40,14 @@ PEAK_TFLOPS = {"f32": 157.3, "bf16": 2516.6}  # MI355X dense MFMA peaks
 PEAK_HBM_GBPS = 8000.0
 METRIC = "MLP fwd+bwd+reduce step ms & TFLOP/s on 1 MI355X; grad-reduce GB/s"
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark
+# (FETCH_SIZE scaled by 1.9986, WRITE_SIZE by 1.0, the factors a plain 33.6 MB device copy gives;
+# the runs are summarised under profiles/).  GEMM: mean over the forward, weight-gradient and
+# input-gradient launches.  None = not measured for that configuration.
+MEASURED_TRAFFIC_BYTES = {
+    "C2": {"gemm": (50.4e6 + 16.8e6 + 151.0e6 + 16.8e6 + 67.2e6 + 16.8e6) / 3, "reduce": 167.8e6 + 33.6e6},
+}
+
 
 def cpu_baseline(nf, B, R, lr, budget_s):
     """Times the CPU restatement of the reference path on this host (rank 0, N = 1 only)."""
@@ -157,12 +165,15 @@ def main():
         "weights_finite": finite,
         "roofline": {"kernel": "gemm_f32_mfma (nt, nn, tn)" if dtype == "f32" else "gemm_bf16_mfma",
                      "bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(gemm_tflops / peak, 4), "traffic": None,
+                     "frac": round(gemm_tflops / peak, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get("gemm") if not args.overlap else None,
                      "flop_per_launch": flop_per_gemm, "avg_launch_us": round(gemm_avg_ms * 1e3, 2),
                      "launches": gemm_launches},
         "roofline_reduce": {"kernel": "reduce_sgd_vec4", "bound": "hbm", "achieved": round(upd_gbps, 1),
                             "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(upd_gbps / PEAK_HBM_GBPS, 4),
-                            "traffic": None, "bytes_per_launch": upd_bytes, "avg_launch_us": round(upd_ms * 1e3, 2)},
+                            "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get("reduce")
+                            if not args.overlap else None,
+                            "bytes_per_launch": upd_bytes, "avg_launch_us": round(upd_ms * 1e3, 2)},
     }
     if args.cpu_seconds > 0:
         out["cpu_baseline"] = cpu_baseline(nf, B, R, args.lr, args.cpu_seconds)
