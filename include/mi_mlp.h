@@ -134,15 +134,35 @@ int mi_reduce_sgd_raw(float* W, const float* G, size_t n, size_t replica_stride,
 int mi_reduce_sgd_bf16_raw(float* W, void* W_bf16, const float* G, size_t n, size_t replica_stride,
                            int R, float lr, void* stream);
 
-/* bf16 variants of the three GEMMs: A, B (and C for nt/nn) are bf16 stored as 16-bit words,
- * products accumulate in fp32.  mi_hgemm_tn writes fp32 gradients. */
+/*
+ * bf16 variants of the three GEMMs (bf16 stored as 16-bit words, fp32 accumulation on
+ * v_mfma_f32_32x32x16_bf16).  A bf16 MFMA reads 8 consecutive k per lane, so every operand must be
+ * K-contiguous; where the fp32 call site reads a row-contiguous operand, the bf16 entry point
+ * takes its transposed copy (mi_transpose_bf16 makes one):
+ *   mi_hgemm_nt  forward          C[M x N] (bf16) = A[M x K] * B[N x K]^T + bias, optional ReLU
+ *   mi_hgemm_nn  input gradient   C[M x N] (bf16) = A[M x K] * B[K x N], given Bt = B^T [N x K],
+ *                                 zeroed where mask_src (bf16, [M x N]) <= 0 if mask_src != NULL
+ *   mi_hgemm_tn  weight gradient  C_r[M x N] (fp32) = A_r^T * B_r over the K rows of replica r,
+ *                                 given At_r = A_r^T [M x K] and Bt_r = B_r^T [N x K]; replica r's
+ *                                 operands start at At + r*strideAt, Bt + r*strideBt (elements)
+ */
 int mi_hgemm_nt(int M, int N, int K, const void* A, int lda, const void* B, int ldb, void* C,
                 int ldc, const float* bias, int relu, void* stream);
-int mi_hgemm_nn(int M, int N, int K, const void* A, int lda, const void* B, int ldb, void* C,
+int mi_hgemm_nn(int M, int N, int K, const void* A, int lda, const void* Bt, int ldbt, void* C,
                 int ldc, const void* mask_src, int ldmask, void* stream);
-int mi_hgemm_tn(int R, int M, int N, int K, const void* A, int lda, const void* B, int ldb,
-                float* C, int ldc, long long strideC, float* colsum, long long stride_colsum,
+int mi_hgemm_tn(int R, int M, int N, int K, const void* At, int ldat, long long strideAt,
+                const void* Bt, int ldbt, long long strideBt, float* C, int ldc, long long strideC,
                 void* stream);
+/* dst[z][c][r] = src[z][r][c] for z < batch: 16-bit elements, leading dimensions and batch
+ * strides in elements. */
+int mi_transpose_bf16(int batch, int rows, int cols, const void* src, int ld_src, long long batch_src,
+                      void* dst, int ld_dst, long long batch_dst, void* stream);
+/* out[z*stride_out + r] = sum over c of src[z][r][c] (fp32 sums of a bf16 matrix): the bias
+ * gradient from a transposed gradient copy. */
+int mi_rowsum_bf16(int batch, int rows, int cols, const void* src, int ld, long long batch_src,
+                   float* out, long long stride_out, void* stream);
+/* Tuning hook for the bf16 kernel, like mi_set_gemm_variant. */
+int mi_set_hgemm_variant(int variant);
 
 /* fp32 <-> bf16 conversion of n contiguous elements on the device. */
 int mi_convert_f32_to_bf16(void* dst_bf16, const float* src, size_t n, void* stream);

@@ -47,8 +47,11 @@ SIGNATURES = {
     "mi_reduce_sgd_bf16_raw": [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_float, c_void_p],
     "mi_hgemm_nt": [c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
     "mi_hgemm_nn": [c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
-    "mi_hgemm_tn": [c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_longlong,
-                    c_void_p, c_longlong, c_void_p],
+    "mi_hgemm_tn": [c_int, c_int, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_int, c_longlong, c_void_p,
+                    c_int, c_longlong, c_void_p],
+    "mi_transpose_bf16": [c_int, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_int, c_longlong, c_void_p],
+    "mi_rowsum_bf16": [c_int, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_longlong, c_void_p],
+    "mi_set_hgemm_variant": [c_int],
     "mi_convert_f32_to_bf16": [c_void_p, c_void_p, c_size_t, c_void_p],
     "mi_convert_bf16_to_f32": [c_void_p, c_void_p, c_size_t, c_void_p],
     "mi_mlp_create": [POINTER(c_void_p), c_int, POINTER(c_int), c_int, c_int, c_int, c_uint],

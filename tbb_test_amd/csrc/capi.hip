@@ -3,6 +3,7 @@
 // and HIP-graph replay.  The arithmetic lives in gemm_f32.hip, gemm_bf16.hip and reduce_sgd.hip.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -43,6 +44,7 @@ int hip_fail(hipError_t e, const char* what) {
   } while (0)
 
 int g_variant[3] = {0, 0, 0};  // forced tile configuration per GEMM kind (nt, nn, tn); 0 = automatic
+int g_hvariant = 0;             // forced tile configuration of the bf16 kernel
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
@@ -64,8 +66,12 @@ struct mi_mlp {
   float* params = nullptr;    // [stride]
   float* grads = nullptr;     // [R * stride]
   uint16_t* params16 = nullptr;  // bf16 copy of params (dtype bf16)
+  uint16_t* params16T = nullptr; // bf16 W_l^T [N_l x N_{l+1}] at the same arena offsets (dtype bf16)
   float* params_saved = nullptr;    // snapshot of params (mi_mlp_snapshot_weights)
   uint16_t* params16_saved = nullptr;
+  uint16_t* params16T_saved = nullptr;
+  std::vector<uint16_t*> actsT;  // bf16 only: per-replica transposed activations [R][N_l x B], l < L
+  uint16_t* dzT = nullptr;       // bf16 only: per-replica transposed gradient [R][max N x B]
   std::vector<void*> acts;    // L+1 buffers [MB x nf[l]], fp32 or bf16
   void* dy = nullptr;         // upstream gradient [MB x nf[L]]
   void* dz[2] = {nullptr, nullptr};  // gradient ping-pong [MB x max width]
@@ -173,7 +179,9 @@ int op_forward(mi_mlp* h, int l, hipStream_t s) {
     e = mi::sgemm_nt(h->MB, h->nf[l + 1], h->nf[l], (const float*)h->acts[l], h->nf[l], h->params + h->woff[l],
                      h->nf[l], (float*)h->acts[l + 1], h->nf[l + 1], h->params + h->boff[l], relu, s, g_variant[0]);
   } else {
-    return fail(MI_ERR_UNSUPPORTED, "bf16 forward is not implemented in this build");
+    e = mi::hgemm_nt(1, h->MB, h->nf[l + 1], h->nf[l], (const uint16_t*)h->acts[l], h->nf[l], 0,
+                     h->params16 + h->woff[l], h->nf[l], 0, h->acts[l + 1], h->nf[l + 1], 0, 1, h->params + h->boff[l],
+                     relu, nullptr, 0, s, g_hvariant);
   }
   if (e != hipSuccess) return hip_fail(e, "forward GEMM launch");
   return ts.finish();
@@ -189,14 +197,33 @@ int op_wgrad(mi_mlp* h, int l, hipStream_t s, bool with_bias) {
                      (const float*)h->acts[l], h->nf[l], const_cast<float*>(g0), h->nf[l], (long long)h->stride,
                      with_bias ? h->grads + h->boff[l] : nullptr, (long long)h->stride, s, g_variant[2]);
   } else {
-    return fail(MI_ERR_UNSUPPORTED, "bf16 weight gradient is not implemented in this build");
+    // K-contiguous copies of both operands, per replica: A_l^T [N_l x B] and dZ_l^T [N_{l+1} x B]
+    const int B = h->B, nin = h->nf[l], nout = h->nf[l + 1];
+    e = mi::transpose_bf16(h->R, B, nin, (const uint16_t*)h->acts[l], nin, (long long)B * nin, h->actsT[l], B,
+                           (long long)nin * B, s);
+    if (e == hipSuccess)
+      e = mi::transpose_bf16(h->R, B, nout, (const uint16_t*)dz_of_layer(h, l), nout, (long long)B * nout, h->dzT, B,
+                             (long long)nout * B, s);
+    if (e == hipSuccess)
+      e = mi::hgemm_nt(h->R, nout, nin, B, h->dzT, B, (long long)nout * B, h->actsT[l], B, (long long)nin * B,
+                       const_cast<float*>(g0), nin, (long long)h->stride, 0, nullptr, 0, nullptr, 0, s, g_hvariant);
+    if (e == hipSuccess && with_bias)
+      e = mi::rowsum_bf16(h->R, nout, B, h->dzT, B, (long long)nout * B, h->grads + h->boff[l], (long long)h->stride, s);
   }
   if (e != hipSuccess) return hip_fail(e, "weight-gradient GEMM launch");
   return ts.finish();
 }
 
 int op_bgrad(mi_mlp* h, int l, hipStream_t s) {
-  if (h->dtype != MI_F32) return fail(MI_ERR_UNSUPPORTED, "bf16 bias gradient is not implemented in this build");
+  if (h->dtype != MI_F32) {
+    const int B = h->B, nout = h->nf[l + 1];
+    hipError_t eb = mi::transpose_bf16(h->R, B, nout, (const uint16_t*)dz_of_layer(h, l), nout, (long long)B * nout,
+                                       h->dzT, B, (long long)nout * B, s);
+    if (eb == hipSuccess)
+      eb = mi::rowsum_bf16(h->R, nout, B, h->dzT, B, (long long)nout * B, h->grads + h->boff[l], (long long)h->stride, s);
+    if (eb != hipSuccess) return hip_fail(eb, "bias-gradient launch");
+    return MI_OK;
+  }
   hipError_t e = mi::colsum_f32(h->R, h->nf[l + 1], h->B, (const float*)dz_of_layer(h, l), h->nf[l + 1],
                                 h->grads + h->boff[l], (long long)h->stride, s);
   if (e != hipSuccess) return hip_fail(e, "bias-gradient launch");
@@ -214,7 +241,9 @@ int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
                      h->params + h->woff[l], h->nf[l], (float*)out, h->nf[l], (const float*)mask, h->nf[l], s,
                      g_variant[1]);
   } else {
-    return fail(MI_ERR_UNSUPPORTED, "bf16 input gradient is not implemented in this build");
+    e = mi::hgemm_nt(1, h->MB, h->nf[l], h->nf[l + 1], (const uint16_t*)dz_of_layer(h, l), h->nf[l + 1], 0,
+                     h->params16T + h->woff[l], h->nf[l + 1], 0, out, h->nf[l], 0, mask ? 2 : 3, nullptr, 0,
+                     (const uint16_t*)mask, h->nf[l], s, g_hvariant);
   }
   if (e != hipSuccess) return hip_fail(e, "input-gradient GEMM launch");
   return ts.finish();
@@ -233,6 +262,13 @@ int op_update(mi_mlp* h, int l_or_all, float lr, hipStream_t s) {
   hipError_t e = mi::reduce_sgd(h->params + off, h->params16 ? h->params16 + off : nullptr, h->grads + off, n,
                                 h->stride, h->R, lr, s);
   if (e != hipSuccess) return hip_fail(e, "reduce+SGD launch");
+  if (h->params16T) {  // refresh the transposed bf16 weight copies the input-gradient GEMMs read
+    const int first = l_or_all >= 0 ? l_or_all : 0, last = l_or_all >= 0 ? l_or_all : h->L - 1;
+    for (int l = first; l <= last && e == hipSuccess; ++l)
+      e = mi::transpose_bf16(1, h->nf[l + 1], h->nf[l], h->params16 + h->woff[l], h->nf[l], 0,
+                             h->params16T + h->woff[l], h->nf[l + 1], 0, s);
+    if (e != hipSuccess) return hip_fail(e, "weight transpose launch");
+  }
   return ts.finish();
 }
 
@@ -448,15 +484,74 @@ int mi_reduce_sgd_bf16_raw(float* W, void* W_bf16, const float* G, size_t n, siz
   return MI_OK;
 }
 
-int mi_hgemm_nt(int, int, int, const void*, int, const void*, int, void*, int, const float*, int, void*) {
-  return fail(MI_ERR_UNSUPPORTED, "bf16 GEMMs are not implemented in this build");
+static int check_hgemm(int M, int N, int K, const void* A, int lda, const void* B, int ldb, const void* C, int ldc) {
+  MI_REQUIRE(M >= 0 && N >= 0 && K >= 0, "negative dimension (M=%d N=%d K=%d)", M, N, K);
+  if (M == 0 || N == 0) return MI_OK;
+  MI_REQUIRE(C != nullptr, "null C");
+  MI_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "null operand");
+  MI_REQUIRE(lda >= K && ldb >= K, "both operands are K-contiguous: lda %d, ldb %d must be >= K %d", lda, ldb, K);
+  MI_REQUIRE(ldc >= N, "ldc %d < N %d", ldc, N);
+  return MI_OK;
 }
-int mi_hgemm_nn(int, int, int, const void*, int, const void*, int, void*, int, const void*, int, void*) {
-  return fail(MI_ERR_UNSUPPORTED, "bf16 GEMMs are not implemented in this build");
+
+int mi_hgemm_nt(int M, int N, int K, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                const float* bias, int relu, void* stream) {
+  if (int rc = check_hgemm(M, N, K, A, lda, B, ldb, C, ldc)) return rc;
+  hipError_t e = mi::hgemm_nt(1, M, N, K, (const uint16_t*)A, lda, 0, (const uint16_t*)B, ldb, 0, C, ldc, 0, 1, bias,
+                              relu, nullptr, 0, as_stream(stream), g_hvariant);
+  if (e != hipSuccess) return hip_fail(e, "mi_hgemm_nt launch");
+  return MI_OK;
 }
-int mi_hgemm_tn(int, int, int, int, const void*, int, const void*, int, float*, int, long long, float*, long long,
-                void*) {
-  return fail(MI_ERR_UNSUPPORTED, "bf16 GEMMs are not implemented in this build");
+
+int mi_hgemm_nn(int M, int N, int K, const void* A, int lda, const void* Bt, int ldbt, void* C, int ldc,
+                const void* mask_src, int ldmask, void* stream) {
+  if (int rc = check_hgemm(M, N, K, A, lda, Bt, ldbt, C, ldc)) return rc;
+  MI_REQUIRE(!mask_src || ldmask >= N, "ldmask %d < N %d", ldmask, N);
+  hipError_t e = mi::hgemm_nt(1, M, N, K, (const uint16_t*)A, lda, 0, (const uint16_t*)Bt, ldbt, 0, C, ldc, 0,
+                              mask_src ? 2 : 3, nullptr, 0, (const uint16_t*)mask_src, ldmask, as_stream(stream),
+                              g_hvariant);
+  if (e != hipSuccess) return hip_fail(e, "mi_hgemm_nn launch");
+  return MI_OK;
+}
+
+int mi_hgemm_tn(int R, int M, int N, int K, const void* At, int ldat, long long strideAt, const void* Bt, int ldbt,
+                long long strideBt, float* C, int ldc, long long strideC, void* stream) {
+  MI_REQUIRE(R >= 0, "negative replica count");
+  if (R == 0) return MI_OK;
+  if (int rc = check_hgemm(M, N, K, At, ldat, Bt, ldbt, C, ldc)) return rc;
+  MI_REQUIRE(R == 1 || strideC >= (long long)(M > 0 ? (size_t)(M - 1) * ldc + N : 0), "strideC overlaps replicas");
+  hipError_t e = mi::hgemm_nt(R, M, N, K, (const uint16_t*)At, ldat, strideAt, (const uint16_t*)Bt, ldbt, strideBt, C,
+                              ldc, strideC, 0, nullptr, 0, nullptr, 0, as_stream(stream), g_hvariant);
+  if (e != hipSuccess) return hip_fail(e, "mi_hgemm_tn launch");
+  return MI_OK;
+}
+
+int mi_transpose_bf16(int batch, int rows, int cols, const void* src, int ld_src, long long batch_src, void* dst,
+                      int ld_dst, long long batch_dst, void* stream) {
+  MI_REQUIRE(batch >= 0 && rows >= 0 && cols >= 0, "negative size");
+  if (batch == 0 || rows == 0 || cols == 0) return MI_OK;
+  MI_REQUIRE(src && dst, "null pointer");
+  MI_REQUIRE(ld_src >= cols && ld_dst >= rows, "leading dimension too small");
+  hipError_t e = mi::transpose_bf16(batch, rows, cols, (const uint16_t*)src, ld_src, batch_src, (uint16_t*)dst, ld_dst,
+                                    batch_dst, as_stream(stream));
+  if (e != hipSuccess) return hip_fail(e, "mi_transpose_bf16 launch");
+  return MI_OK;
+}
+
+int mi_rowsum_bf16(int batch, int rows, int cols, const void* src, int ld, long long batch_src, float* out,
+                   long long stride_out, void* stream) {
+  MI_REQUIRE(batch >= 0 && rows >= 0 && cols >= 0, "negative size");
+  if (batch == 0 || rows == 0) return MI_OK;
+  MI_REQUIRE(out && (cols == 0 || src), "null pointer");
+  hipError_t e = mi::rowsum_bf16(batch, rows, cols, (const uint16_t*)src, ld, batch_src, out, stride_out,
+                                 as_stream(stream));
+  if (e != hipSuccess) return hip_fail(e, "mi_rowsum_bf16 launch");
+  return MI_OK;
+}
+
+int mi_set_hgemm_variant(int variant) {
+  g_hvariant = variant;
+  return MI_OK;
 }
 
 int mi_convert_f32_to_bf16(void* dst, const float* src, size_t n, void* stream) {
@@ -484,7 +579,8 @@ int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_repli
   MI_REQUIRE((long long)batch_per_replica * R <= 0x7fffffffLL, "R * batch overflows int");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "unknown dtype %d", dtype);
   for (int l = 0; l <= L; ++l) MI_REQUIRE(nfeatures[l] >= 1, "nfeatures[%d] = %d must be positive", l, nfeatures[l]);
-  if (dtype == MI_BF16) return fail(MI_ERR_UNSUPPORTED, "the bf16 model is not implemented in this build");
+  if (dtype == MI_BF16 && (flags & MI_FLAG_RELU_LAST))
+    return fail(MI_ERR_UNSUPPORTED, "MI_FLAG_RELU_LAST is not implemented for bf16 models");
 
   int count = 0;
   if (hipGetDeviceCount(&count) != hipSuccess || count == 0) return fail(MI_ERR_NO_DEVICE, "no HIP device visible");
@@ -523,6 +619,17 @@ int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_repli
   const size_t es = h->esize();
   alloc((void**)&h->params, h->stride * 4);
   alloc((void**)&h->grads, h->stride * 4 * (size_t)R);
+  if (dtype == MI_BF16) {
+    alloc((void**)&h->params16, h->stride * 2);
+    alloc((void**)&h->params16T, h->stride * 2);
+    h->actsT.assign(L, nullptr);
+    for (int l = 0; l < L; ++l) alloc((void**)&h->actsT[l], (size_t)h->MB * h->nf[l] * 2);
+    alloc((void**)&h->dzT, (size_t)h->MB * h->maxw() * 2);
+    size_t wmax = 0;
+    for (int l = 0; l < L; ++l) wmax = std::max(wmax, (size_t)h->nf[l] * h->nf[l + 1]);
+    h->staging_elems = std::max((size_t)h->MB * h->maxw(), wmax);
+    alloc((void**)&h->staging, h->staging_elems * 4);
+  }
   h->acts.assign(L + 1, nullptr);
   for (int l = 0; l <= L; ++l) alloc(&h->acts[l], (size_t)h->MB * h->nf[l] * es);
   alloc(&h->dy, (size_t)h->MB * h->nf[L] * es);
@@ -570,6 +677,10 @@ int mi_mlp_destroy(mi_mlp* h) {
   (void)hipFree(h->params16);
   (void)hipFree(h->params_saved);
   (void)hipFree(h->params16_saved);
+  (void)hipFree(h->params16T);
+  (void)hipFree(h->params16T_saved);
+  for (auto a : h->actsT) (void)hipFree(a);
+  (void)hipFree(h->dzT);
   for (void* a : h->acts) (void)hipFree(a);
   (void)hipFree(h->dy);
   (void)hipFree(h->dz[0]);
@@ -589,6 +700,15 @@ int mi_mlp_set_weights(mi_mlp* h, int l, const float* W, int ld, const float* b)
     MI_HIP(hipMemcpy(h->params + h->boff[l], b, (size_t)h->nf[l + 1] * 4, hipMemcpyHostToDevice));
   } else {
     MI_HIP(hipMemsetAsync(h->params + h->boff[l], 0, (size_t)h->nf[l + 1] * 4, h->stream));
+    MI_HIP(hipStreamSynchronize(h->stream));
+  }
+  if (h->params16) {
+    const size_t n = (size_t)h->nf[l + 1] * h->nf[l];
+    hipError_t e = mi::convert_f32_to_bf16(h->params16 + h->woff[l], h->params + h->woff[l], n, h->stream);
+    if (e == hipSuccess)
+      e = mi::transpose_bf16(1, h->nf[l + 1], h->nf[l], h->params16 + h->woff[l], h->nf[l], 0,
+                             h->params16T + h->woff[l], h->nf[l + 1], 0, h->stream);
+    if (e != hipSuccess) return hip_fail(e, "bf16 weight copy");
     MI_HIP(hipStreamSynchronize(h->stream));
   }
   return MI_OK;
@@ -707,7 +827,9 @@ int mi_mlp_snapshot_weights(mi_mlp* h) {
   MI_HIP(hipMemcpyAsync(h->params_saved, h->params, h->stride * 4, hipMemcpyDeviceToDevice, h->stream));
   if (h->params16) {
     if (!h->params16_saved) MI_HIP(hipMalloc((void**)&h->params16_saved, h->stride * 2));
+    if (!h->params16T_saved) MI_HIP(hipMalloc((void**)&h->params16T_saved, h->stride * 2));
     MI_HIP(hipMemcpyAsync(h->params16_saved, h->params16, h->stride * 2, hipMemcpyDeviceToDevice, h->stream));
+    MI_HIP(hipMemcpyAsync(h->params16T_saved, h->params16T, h->stride * 2, hipMemcpyDeviceToDevice, h->stream));
   }
   return MI_OK;
 }
@@ -716,8 +838,10 @@ int mi_mlp_restore_weights(mi_mlp* h) {
   if (int rc = check_handle(h)) return rc;
   MI_REQUIRE(h->params_saved != nullptr, "no snapshot taken");
   MI_HIP(hipMemcpyAsync(h->params, h->params_saved, h->stride * 4, hipMemcpyDeviceToDevice, h->stream));
-  if (h->params16)
+  if (h->params16) {
     MI_HIP(hipMemcpyAsync(h->params16, h->params16_saved, h->stride * 2, hipMemcpyDeviceToDevice, h->stream));
+    MI_HIP(hipMemcpyAsync(h->params16T, h->params16T_saved, h->stride * 2, hipMemcpyDeviceToDevice, h->stream));
+  }
   return MI_OK;
 }
 

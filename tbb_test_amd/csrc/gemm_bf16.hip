@@ -1,2 +1,334 @@
-// bf16 GEMM kernels (placeholder translation unit; the kernels are added with the bf16 model).
+// bf16 GEMM for gfx950 on v_mfma_f32_32x32x16_bf16 (fp32 accumulation), plus the helpers the
+// bf16 model needs around it (tiled transpose, row sums).
+//
+// One kernel shape serves all three GEMMs of the MLP step: C[M,N] = A[M,K] * B[N,K]^T with both
+// operands K-contiguous.  A bf16 MFMA wants 8 consecutive k per lane for its row, so an operand
+// whose rows are contiguous instead (B of the input-gradient GEMM, both operands of the weight
+// gradient) would have to be transposed on its way into the registers; here the handle keeps
+// K-contiguous bf16 copies instead (W^T next to W, A_l^T and dZ_l^T next to A_l and dZ_l, written
+// by transpose_bf16) -- at the sizes the bf16 path is for, a transpose moves a few hundred MB
+// while the GEMM it feeds does TFLOPs:
+//   forward          Y   = X    * W^T            A = X,       B = W
+//   input gradient   dA  = dZ   * W = dZ * (W^T)^T   A = dZ,  B = W^T
+//   weight gradient  dW_r = dZ_r^T * A_r         A = dZ_r^T,  B = A_r^T      (reference call sites
+//                                                mlp_omp.cc:474-488, 657-671, 565-580)
+//
+// Structure: as the fp32 kernel -- three LDS buffers, tile t+1 written to LDS at the top of step
+// t, loads of tile t+2 issued right after, one LDS-only barrier in the middle of the step,
+// operand fragments of the next 16-wide K chunk fetched while the current chunk is multiplied.
+// Tiles are stored [row][BK + 8] (16-byte pad per row); a lane fetches its 8 k values of one
+// 32 x 32 block with one 16-byte LDS read.
+#include <hip/hip_runtime.h>
+
 #include "kernels.h"
+
+namespace mi {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned short u16;
+
+enum EpilogueH { EPH_F32 = 0, EPH_BIAS_RELU = 1, EPH_MASK = 2, EPH_BF16 = 3 };
+
+struct HGemmArgs {
+  int M, N, K;
+  const u16* A;
+  const u16* B;
+  void* C;  // bf16 or fp32, see the epilogue
+  int lda, ldb, ldc;
+  long long batchA, batchB, batchC;  // element offsets per blockIdx.z
+  const float* bias;
+  int relu;
+  const u16* mask;  // bf16 [M x N]: result zeroed where mask <= 0
+  int ldmask;
+  int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ u16 f2bf(float f) {
+  unsigned int u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (u16)(u >> 16);
+}
+__device__ __forceinline__ float bf2f(u16 h) { return __uint_as_float((unsigned int)h << 16); }
+
+__device__ __forceinline__ void lds_barrier_h() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int EPI>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int STRIDE = BK + 8;                 // bf16 elements per LDS row
+  constexpr int A_ELEMS = BM * STRIDE, B_ELEMS = BN * STRIDE;
+  constexpr int VPR = BK / 8;                    // 16-byte vectors per tile row
+  constexpr int NVA = BM * VPR / NT, NVB = BN * VPR / NT;
+  constexpr int CH = BK / 16;                    // 16-wide K chunks per step
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 16 == 0, "tile shape");
+  static_assert((BM * VPR) % NT == 0 && (BN * VPR) % NT == 0, "tile must divide over the threads");
+  static_assert(CH % 2 == 0, "two fragment sets alternate per chunk");
+
+  extern __shared__ __attribute__((aligned(16))) u16 smem_h[];
+  auto As = [&](int buf) { return smem_h + buf * A_ELEMS; };
+  auto Bs = [&](int buf) { return smem_h + 3 * A_ELEMS + buf * B_ELEMS; };
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hi = lane >> 5;
+  const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
+
+  // XCD-aware tile order: XCD x (workgroup id % 8) gets a contiguous range of the row-major
+  // tile order, so tiles that share an A panel share an L2
+  int id = blockIdx.x;
+  const int total = p.tiles_m * p.tiles_n;
+  if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+  const int tile_m = id / p.tiles_n, tile_n = id - tile_m * p.tiles_n;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const u16* __restrict__ a_ptr = p.A + (size_t)blockIdx.z * p.batchA + (size_t)m0 * p.lda;
+  const u16* __restrict__ b_ptr = p.B + (size_t)blockIdx.z * p.batchB + (size_t)n0 * p.ldb;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  u32x4 ra[NVA], rb[NVB];
+  auto fetch = [&]() {
+#pragma unroll
+    for (int i = 0; i < NVA; ++i) {
+      const int idx = tid + i * NT, row = idx / VPR, c = idx % VPR;
+      ra[i] = *reinterpret_cast<const u32x4*>(a_ptr + (size_t)row * p.lda + c * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < NVB; ++i) {
+      const int idx = tid + i * NT, row = idx / VPR, c = idx % VPR;
+      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (size_t)row * p.ldb + c * 8);
+    }
+    a_ptr += BK;
+    b_ptr += BK;
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < NVA; ++i) {
+      const int idx = tid + i * NT, row = idx / VPR, c = idx % VPR;
+      *reinterpret_cast<u32x4*>(As(buf) + row * STRIDE + c * 8) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NVB; ++i) {
+      const int idx = tid + i * NT, row = idx / VPR, c = idx % VPR;
+      *reinterpret_cast<u32x4*>(Bs(buf) + row * STRIDE + c * 8) = rb[i];
+    }
+  };
+  auto load_frags = [&](bf16x8 (&fa)[TM], bf16x8 (&fb)[TN], int buf, int kk) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      fa[i] = *reinterpret_cast<const bf16x8*>(As(buf) + (wm0 + i * 32 + l32) * STRIDE + kk * 16 + hi * 8);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      fb[j] = *reinterpret_cast<const bf16x8*>(Bs(buf) + (wn0 + j * 32 + l32) * STRIDE + kk * 16 + hi * 8);
+  };
+
+  const int nk = p.K / BK;
+  fetch();
+  stash(0);
+  if (nk > 1) fetch();
+  lds_barrier_h();
+  bf16x8 fa[2][TM], fb[2][TN];
+  load_frags(fa[0], fb[0], 0, 0);
+  int cur = 0;
+  for (int t = 0; t < nk; ++t) {
+    const int nxt = cur == 2 ? 0 : cur + 1;
+#pragma unroll
+    for (int kk = 0; kk < CH; ++kk) {
+      const int fc = kk & 1, fn = fc ^ 1;
+      if (kk + 1 < CH) load_frags(fa[fn], fb[fn], cur, kk + 1);
+      else if (t + 1 < nk) load_frags(fa[fn], fb[fn], nxt, 0);
+      if (kk == 0) {
+        if (t + 1 < nk) stash(nxt);
+        if (t + 2 < nk) fetch();
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[fc][i], fb[fc][j], acc[i][j], 0, 0, 0);
+      if (kk == CH - 2) lds_barrier_h();
+    }
+    cur = nxt;
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------------
+  const int col0 = n0 + wn0 + l32;
+  float bias_v[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) bias_v[j] = (EPI == EPH_BIAS_RELU && p.bias) ? p.bias[col0 + j * 32] : 0.0f;
+  float* __restrict__ cf = reinterpret_cast<float*>(p.C) + (size_t)blockIdx.z * p.batchC;
+  u16* __restrict__ ch = reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = col0 + j * 32;
+        float v = acc[i][j][r];
+        if (EPI == EPH_F32) {
+          cf[(size_t)row * p.ldc + col] = v;
+        } else {
+          if (EPI == EPH_BIAS_RELU) {
+            v += bias_v[j];
+            if (p.relu) v = v > 0.0f ? v : 0.0f;
+          } else if (EPI == EPH_MASK) {
+            if (!(bf2f(p.mask[(size_t)row * p.ldmask + col]) > 0.0f)) v = 0.0f;
+          }
+          ch[(size_t)row * p.ldc + col] = f2bf(v);
+        }
+      }
+    }
+  }
+}
+
+// Any-shape fallback: one thread per output element, fp32 accumulation in k order.
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_generic(HGemmArgs p) {
+  const int col = blockIdx.x * 16 + (threadIdx.x & 15), row = blockIdx.y * 16 + (threadIdx.x >> 4);
+  if (row >= p.M || col >= p.N) return;
+  const u16* a = p.A + (size_t)blockIdx.z * p.batchA + (size_t)row * p.lda;
+  const u16* b = p.B + (size_t)blockIdx.z * p.batchB + (size_t)col * p.ldb;
+  float v = 0.0f;
+  for (int k = 0; k < p.K; ++k) v = fmaf(bf2f(a[k]), bf2f(b[k]), v);
+  if (EPI == EPH_F32) {
+    (reinterpret_cast<float*>(p.C) + (size_t)blockIdx.z * p.batchC)[(size_t)row * p.ldc + col] = v;
+    return;
+  }
+  if (EPI == EPH_BIAS_RELU) {
+    if (p.bias) v += p.bias[col];
+    if (p.relu) v = v > 0.0f ? v : 0.0f;
+  } else if (EPI == EPH_MASK) {
+    if (!(bf2f(p.mask[(size_t)row * p.ldmask + col]) > 0.0f)) v = 0.0f;
+  }
+  (reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC)[(size_t)row * p.ldc + col] = f2bf(v);
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int EPI>
+static hipError_t launch_h(HGemmArgs& p, int batch, hipStream_t s) {
+  constexpr size_t lds_bytes = 3 * (size_t)(BM + BN) * (BK + 8) * sizeof(u16);
+  auto kern = gemm_bf16_mfma<BM, BN, BK, WM, WN, EPI>;
+  static bool attr_set = false;
+  if (lds_bytes > 64 * 1024 && !attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  p.tiles_m = p.M / BM;
+  p.tiles_n = p.N / BN;
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
+  return hipGetLastError();
+}
+
+template <int EPI>
+static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant) {
+  if (p.M <= 0 || p.N <= 0 || batch <= 0) return hipSuccess;
+  auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  const bool vec_ok = al16(p.A) && al16(p.B) && p.lda % 8 == 0 && p.ldb % 8 == 0 && p.batchA % 8 == 0 &&
+                      p.batchB % 8 == 0 && p.K > 0;
+  auto fits = [&](int bm, int bn, int bk) { return vec_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0; };
+  if (variant == 0) {
+    const long long t256 = (long long)(p.M / 256) * (p.N / 256) * batch;
+    if (fits(256, 256, 32) && t256 >= 256) variant = 1;
+    else if (fits(128, 128, 32)) variant = 3;
+    else if (fits(64, 64, 32)) variant = 5;
+    else variant = -1;
+  }
+  switch (variant) {
+    case 1: if (fits(256, 256, 32)) return launch_h<256, 256, 32, 2, 2, EPI>(p, batch, s); break;
+    case 2: if (fits(256, 128, 32)) return launch_h<256, 128, 32, 2, 2, EPI>(p, batch, s); break;
+    case 3: if (fits(128, 128, 32)) return launch_h<128, 128, 32, 2, 2, EPI>(p, batch, s); break;
+    case 4: if (fits(256, 256, 32)) return launch_h<256, 256, 32, 2, 4, EPI>(p, batch, s); break;
+    case 5: if (fits(64, 64, 32)) return launch_h<64, 64, 32, 2, 2, EPI>(p, batch, s); break;
+    case 6: if (fits(128, 128, 64)) return launch_h<128, 128, 64, 2, 2, EPI>(p, batch, s); break;
+    default: break;
+  }
+  hipLaunchKernelGGL((gemm_bf16_generic<EPI>), dim3((p.N + 15) / 16, (p.M + 15) / 16, batch), dim3(256), 0, s, p);
+  return hipGetLastError();
+}
+
+// C = A[M,K] * B[N,K]^T, both bf16 and K-contiguous.  out_kind: 0 fp32 plain, 1 bf16 bias+ReLU,
+// 2 bf16 masked, 3 bf16 plain.
+hipError_t hgemm_nt(int batch, int M, int N, int K, const uint16_t* A, int lda, long long batchA, const uint16_t* B,
+                    int ldb, long long batchB, void* C, int ldc, long long batchC, int out_kind, const float* bias,
+                    int relu, const uint16_t* mask, int ldmask, hipStream_t s, int variant) {
+  HGemmArgs p{};
+  p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+  p.batchA = batchA; p.batchB = batchB; p.batchC = batchC;
+  p.bias = bias; p.relu = relu; p.mask = mask; p.ldmask = ldmask;
+  switch (out_kind) {
+    case 0: return dispatch_h<EPH_F32>(p, batch, s, variant);
+    case 1: return dispatch_h<EPH_BIAS_RELU>(p, batch, s, variant);
+    case 2: return dispatch_h<EPH_MASK>(p, batch, s, variant);
+    default: return dispatch_h<EPH_BF16>(p, batch, s, variant);
+  }
+}
+
+// ---- batched transpose: dst[z][c][r] = src[z][r][c], 16-bit elements, 64 x 64 tiles through LDS ----
+__global__ __launch_bounds__(256) void transpose16_kernel(u16* __restrict__ dst, const u16* __restrict__ src, int rows,
+                                                          int cols, int ld_src, int ld_dst, long long batch_src,
+                                                          long long batch_dst) {
+  __shared__ u16 tile[64][66];
+  const u16* s = src + (size_t)blockIdx.z * batch_src;
+  u16* d = dst + (size_t)blockIdx.z * batch_dst;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int r = r0 + i, c = c0 + tx;
+    tile[i][tx] = (r < rows && c < cols) ? s[(size_t)r * ld_src + c] : (u16)0;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int c = c0 + i, r = r0 + tx;
+    if (c < cols && r < rows) d[(size_t)c * ld_dst + r] = tile[tx][i];
+  }
+}
+
+hipError_t transpose_bf16(int batch, int rows, int cols, const uint16_t* src, int ld_src, long long batch_src,
+                          uint16_t* dst, int ld_dst, long long batch_dst, hipStream_t s) {
+  if (batch <= 0 || rows <= 0 || cols <= 0) return hipSuccess;
+  hipLaunchKernelGGL(transpose16_kernel, dim3((cols + 63) / 64, (rows + 63) / 64, batch), dim3(256), 0, s, dst, src, rows,
+                     cols, ld_src, ld_dst, batch_src, batch_dst);
+  return hipGetLastError();
+}
+
+// ---- row sums of a bf16 matrix in fp32: out[z*stride_out + r] = sum_c src[z][r][c] -------------------
+// One wavefront per row, lanes stride over the columns, fixed-order tree at the end.
+__global__ __launch_bounds__(256) void rowsum16_kernel(float* __restrict__ out, const u16* __restrict__ src, int rows,
+                                                       int cols, int ld, long long batch_src, long long stride_out) {
+  const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const u16* s = src + (size_t)blockIdx.y * batch_src + (size_t)row * ld;
+  float v = 0.0f;
+  for (int c = lane; c < cols; c += 64) v += bf2f(s[c]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  if (lane == 0) out[(size_t)blockIdx.y * stride_out + row] = v;
+}
+
+hipError_t rowsum_bf16(int batch, int rows, int cols, const uint16_t* src, int ld, long long batch_src, float* out,
+                       long long stride_out, hipStream_t s) {
+  if (batch <= 0 || rows <= 0) return hipSuccess;
+  hipLaunchKernelGGL(rowsum16_kernel, dim3((rows + 3) / 4, batch), dim3(256), 0, s, out, src, rows, cols, ld, batch_src,
+                     stride_out);
+  return hipGetLastError();
+}
+
+}  // namespace mi

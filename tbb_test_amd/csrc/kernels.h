@@ -28,6 +28,19 @@ hipError_t colsum_f32(int R, int M, int K, const float* A, int lda, float* out, 
 hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t stride, int R, float lr,
                       hipStream_t s);
 
+// bf16: C = A[M,K] * B[N,K]^T with fp32 accumulation, both operands K-contiguous, blockIdx.z
+// batches with element strides batchA/B/C.  out_kind: 0 fp32 plain, 1 bf16 with bias + optional
+// ReLU, 2 bf16 zeroed where mask (bf16) <= 0, 3 bf16 plain.
+hipError_t hgemm_nt(int batch, int M, int N, int K, const uint16_t* A, int lda, long long batchA, const uint16_t* B,
+                    int ldb, long long batchB, void* C, int ldc, long long batchC, int out_kind, const float* bias,
+                    int relu, const uint16_t* mask, int ldmask, hipStream_t s, int variant);
+// dst[z][c][r] = src[z][r][c] for 16-bit elements
+hipError_t transpose_bf16(int batch, int rows, int cols, const uint16_t* src, int ld_src, long long batch_src,
+                          uint16_t* dst, int ld_dst, long long batch_dst, hipStream_t s);
+// out[z*stride_out + r] = sum_c src[z][r][c] in fp32
+hipError_t rowsum_bf16(int batch, int rows, int cols, const uint16_t* src, int ld, long long batch_src, float* out,
+                       long long stride_out, hipStream_t s);
+
 hipError_t convert_f32_to_bf16(uint16_t* dst, const float* src, size_t n, hipStream_t s);
 hipError_t convert_bf16_to_f32(float* dst, const uint16_t* src, size_t n, hipStream_t s);
 

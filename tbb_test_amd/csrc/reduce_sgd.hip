@@ -23,33 +23,61 @@ __device__ __forceinline__ unsigned short f32_to_bf16_rne(float f) {
   return (unsigned short)(u >> 16);
 }
 
-// One float4 per thread per trip; UNROLL independent trips in flight.  The gradients are read
-// exactly once, so they are loaded non-temporally; W is read and rewritten in place.
-template <int R_FIXED, bool WRITE_BF16>
+// UNROLL float4 per thread per trip.  Two regimes, chosen by the launcher from the bytes moved:
+//   STREAM = true   the arenas exceed the 256 MB Infinity Cache: the gradients are read exactly
+//                   once, so they are loaded non-temporally; one float4 per thread, one trip.
+//   STREAM = false  everything fits the Infinity Cache, where the gradient GEMMs have just left
+//                   their output: ordinary loads (non-temporal ones would bypass that cache), two
+//                   float4 per thread in flight.
+template <int R_FIXED, bool WRITE_BF16, int UNROLL, bool STREAM>
 __global__ __launch_bounds__(256) void reduce_sgd_vec4(float* __restrict__ W, unsigned short* __restrict__ W16,
                                                        const float* __restrict__ G, size_t nvec,
                                                        size_t stride_vec, int R_dyn, float neg_lr) {
   const int R = R_FIXED > 0 ? R_FIXED : R_dyn;
   const f32x4* __restrict__ g4 = reinterpret_cast<const f32x4*>(G);
   f32x4* __restrict__ w4 = reinterpret_cast<f32x4*>(W);
-  const size_t step = (size_t)gridDim.x * blockDim.x;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += step) {
-    f32x4 s = __builtin_nontemporal_load(g4 + i);
+  auto ld = [&](const f32x4* ptr) { return STREAM ? __builtin_nontemporal_load(ptr) : *ptr; };
+  const size_t step = (size_t)gridDim.x * blockDim.x * UNROLL;
+  for (size_t base = (size_t)blockIdx.x * blockDim.x * UNROLL + threadIdx.x; base < nvec; base += step) {
+    f32x4 s[UNROLL], w[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const size_t i = base + (size_t)u * blockDim.x;
+      if (i < nvec) {
+        s[u] = ld(g4 + i);
+        w[u] = w4[i];
+      }
+    }
     if (R_FIXED > 0) {
 #pragma unroll
-      for (int r = 1; r < R_FIXED; ++r) s += __builtin_nontemporal_load(g4 + (size_t)r * stride_vec + i);
+      for (int r = 1; r < R_FIXED; ++r)
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+          const size_t i = base + (size_t)u * blockDim.x;
+          if (i < nvec) s[u] += ld(g4 + (size_t)r * stride_vec + i);
+        }
     } else {
-      for (int r = 1; r < R; ++r) s += __builtin_nontemporal_load(g4 + (size_t)r * stride_vec + i);
+      for (int r = 1; r < R; ++r)
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+          const size_t i = base + (size_t)u * blockDim.x;
+          if (i < nvec) s[u] += ld(g4 + (size_t)r * stride_vec + i);
+        }
     }
-    f32x4 w = w4[i];
-    w[0] = fmaf(neg_lr, s[0], w[0]);
-    w[1] = fmaf(neg_lr, s[1], w[1]);
-    w[2] = fmaf(neg_lr, s[2], w[2]);
-    w[3] = fmaf(neg_lr, s[3], w[3]);
-    w4[i] = w;
-    if (WRITE_BF16) {
-      u16x4 h = {f32_to_bf16_rne(w[0]), f32_to_bf16_rne(w[1]), f32_to_bf16_rne(w[2]), f32_to_bf16_rne(w[3])};
-      reinterpret_cast<u16x4*>(W16)[i] = h;
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const size_t i = base + (size_t)u * blockDim.x;
+      if (i >= nvec) continue;
+      f32x4 o;
+      o[0] = fmaf(neg_lr, s[u][0], w[u][0]);
+      o[1] = fmaf(neg_lr, s[u][1], w[u][1]);
+      o[2] = fmaf(neg_lr, s[u][2], w[u][2]);
+      o[3] = fmaf(neg_lr, s[u][3], w[u][3]);
+      w4[i] = o;
+      if (WRITE_BF16) {
+        u16x4 h = {f32_to_bf16_rne(o[0]), f32_to_bf16_rne(o[1]), f32_to_bf16_rne(o[2]), f32_to_bf16_rne(o[3])};
+        reinterpret_cast<u16x4*>(W16)[i] = h;
+      }
     }
   }
 }
@@ -84,11 +112,19 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
   size_t done = 0;
   if (vec && n >= 4) {
     const size_t nvec = n / 4;
-    // 256 CUs x 8 resident workgroups of 256 threads covers the chip; more only adds launch work
-    const int blocks = grid_for(nvec, 256, 256 * 8);
-#define MI_LAUNCH_REDUCE(RF, BF)                                                                       \
-  hipLaunchKernelGGL((reduce_sgd_vec4<RF, BF>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, stride / 4, \
-                     R, neg_lr)
+    const bool stream = (double)(R + 1) * (double)n * 4.0 > 192e6;  // beyond what the Infinity Cache holds
+    const size_t per_block = stream ? 256 : 512;
+    const int blocks = grid_for(nvec, (int)per_block, stream ? (1 << 30) : 8192);
+#define MI_LAUNCH_REDUCE2(RF, BF)                                                                          \
+  do {                                                                                                     \
+    if (stream)                                                                                            \
+      hipLaunchKernelGGL((reduce_sgd_vec4<RF, BF, 1, true>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, \
+                         stride / 4, R, neg_lr);                                                           \
+    else                                                                                                   \
+      hipLaunchKernelGGL((reduce_sgd_vec4<RF, BF, 2, false>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, \
+                         stride / 4, R, neg_lr);                                                           \
+  } while (0)
+#define MI_LAUNCH_REDUCE(RF, BF) MI_LAUNCH_REDUCE2(RF, BF)
     if (W16) {
       switch (R) {
         case 1: MI_LAUNCH_REDUCE(1, true); break;
@@ -106,6 +142,7 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
         default: MI_LAUNCH_REDUCE(0, false); break;
       }
     }
+#undef MI_LAUNCH_REDUCE2
 #undef MI_LAUNCH_REDUCE
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

@@ -1,0 +1,198 @@
+"""GPU parity of the bf16 path (bf16 operands, fp32 MFMA accumulation, fp32 master weights and
+gradients) against the fp32 CPU oracle.  Bound: rel-err <= 2e-2 (max|a-e| / max|e|).  Raw GEMMs
+are fed bf16-representable inputs, so their only error is the accumulation order and the final
+rounding of the output to bf16 (2^-9 relative); their bound is tighter and stated per test."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oracle
+from conftest import BF16_TOL, rel_err
+from tbb_test_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+
+def to_bf16_bits(a):
+    """fp32 -> bf16 bit pattern, round to nearest even (numpy restatement of the device rounding)."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    u = u + 0x7FFF + ((u >> 16) & 1)
+    return (u >> 16).astype(np.uint16)
+
+
+def from_bf16_bits(h):
+    return (np.asarray(h, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def bf16_round(a):
+    return from_bf16_bits(to_bf16_bits(a))
+
+
+def dev16(a):
+    return capi.DeviceBuffer.from_numpy(to_bf16_bits(a))
+
+
+def test_bf16_helpers_round_to_nearest_even():
+    x = np.array([1.0, 1.0 + 2 ** -8, 1.0 + 2 ** -7 + 2 ** -8, -3.140625, 1e-30], np.float32)
+    got = bf16_round(x)
+    assert got[0] == 1.0 and got[1] == 1.0 and got[2] == np.float32(1.0 + 2 ** -6) and got[3] == np.float32(-3.140625)
+    # the device conversion kernel agrees bit for bit
+    rng = np.random.default_rng(0)
+    v = rng.standard_normal(100003).astype(np.float32)
+    src = capi.DeviceBuffer.from_numpy(v)
+    dst = capi.DeviceBuffer(v.size * 2)
+    lib = capi.lib()
+    capi.check(lib.mi_convert_f32_to_bf16(dst.ptr, src.ptr, v.size, None))
+    back = capi.DeviceBuffer(v.size * 4)
+    capi.check(lib.mi_convert_bf16_to_f32(back.ptr, dst.ptr, v.size, None))
+    capi.check(lib.mi_stream_sync(None))
+    assert np.array_equal(dst.to_numpy((v.size,), np.uint16), to_bf16_bits(v))
+    assert np.array_equal(back.to_numpy((v.size,)), bf16_round(v))
+
+
+HSHAPES = [(64, 64, 32), (128, 128, 64), (256, 256, 96), (512, 256, 128), (256, 512, 32), (7, 5, 9), (100, 130, 50),
+           (129, 64, 40)]
+HVARIANTS = [0, 1, 2, 3, 4, 5, 6]
+
+
+@pytest.mark.parametrize("variant", HVARIANTS)
+@pytest.mark.parametrize("shape", HSHAPES)
+def test_hgemm_forward_and_input_gradient(shape, variant):
+    M, N, K = shape
+    rng = np.random.default_rng(M + 3 * N + 5 * K)
+    A = bf16_round(rng.uniform(-1, 1, (M, K)))
+    B = bf16_round(rng.uniform(-1, 1, (N, K)))
+    bias = rng.uniform(-1, 1, N).astype(np.float32)
+    act = bf16_round(np.maximum(rng.uniform(-1, 1, (M, N)), 0))
+    lib = capi.lib()
+    dA, dB, dbias, dact = dev16(A), dev16(B), capi.DeviceBuffer.from_numpy(bias), dev16(act)
+    dC = capi.DeviceBuffer(M * N * 2)
+    capi.check(lib.mi_set_hgemm_variant(variant))
+    try:
+        capi.check(lib.mi_hgemm_nt(M, N, K, dA.ptr, K, dB.ptr, K, dC.ptr, N, dbias.ptr, 1, None))
+        capi.check(lib.mi_stream_sync(None))
+        got = from_bf16_bits(dC.to_numpy((M, N), np.uint16))
+        assert rel_err(got, oracle.fc_forward(A, B, bias, True)) <= 4e-3, (shape, variant)
+        # input gradient: C = A * Bt^T with the mask; the oracle takes the untransposed weight
+        capi.check(lib.mi_hgemm_nn(M, N, K, dA.ptr, K, dB.ptr, K, dC.ptr, N, dact.ptr, N, None))
+        capi.check(lib.mi_stream_sync(None))
+        got = from_bf16_bits(dC.to_numpy((M, N), np.uint16))
+        want = oracle.fc_dgrad(A, np.ascontiguousarray(B.T), act)
+        assert rel_err(got, want) <= 4e-3, (shape, variant)
+        assert np.all(got[act <= 0] == 0.0)
+    finally:
+        lib.mi_set_hgemm_variant(0)
+
+
+@pytest.mark.parametrize("variant", HVARIANTS)
+@pytest.mark.parametrize("R", [1, 3])
+@pytest.mark.parametrize("shape", HSHAPES)
+def test_hgemm_weight_gradient_via_transposed_copies(shape, R, variant):
+    """dW_r = dZ_r^T A_r computed from the K-contiguous copies dZ_r^T, A_r^T that
+    mi_transpose_bf16 makes; fp32 output; bias gradient from mi_rowsum_bf16."""
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K + R)
+    dZ = bf16_round(rng.standard_normal((R * K, M)))
+    A = bf16_round(rng.uniform(-1, 1, (R * K, N)))
+    lib = capi.lib()
+    d_dz, d_a = dev16(dZ), dev16(A)
+    d_dzT, d_aT = capi.DeviceBuffer(R * M * K * 2), capi.DeviceBuffer(R * N * K * 2)
+    dC = capi.DeviceBuffer(R * M * N * 4)
+    dS = capi.DeviceBuffer(R * M * 4)
+    capi.check(lib.mi_transpose_bf16(R, K, M, d_dz.ptr, M, K * M, d_dzT.ptr, K, M * K, None))
+    capi.check(lib.mi_transpose_bf16(R, K, N, d_a.ptr, N, K * N, d_aT.ptr, K, N * K, None))
+    capi.check(lib.mi_set_hgemm_variant(variant))
+    try:
+        capi.check(lib.mi_hgemm_tn(R, M, N, K, d_dzT.ptr, K, M * K, d_aT.ptr, K, N * K, dC.ptr, N, M * N, None))
+    finally:
+        lib.mi_set_hgemm_variant(0)
+    capi.check(lib.mi_rowsum_bf16(R, M, K, d_dzT.ptr, K, M * K, dS.ptr, M, None))
+    capi.check(lib.mi_stream_sync(None))
+    assert np.array_equal(d_dzT.to_numpy((R, M, K), np.uint16),
+                          to_bf16_bits(dZ).reshape(R, K, M).transpose(0, 2, 1))  # the transpose is exact
+    C = dC.to_numpy((R, M, N))
+    S = dS.to_numpy((R, M))
+    for r in range(R):
+        dW, db = oracle.fc_wgrad(dZ[r * K:(r + 1) * K], A[r * K:(r + 1) * K])
+        assert rel_err(C[r], dW) <= 1e-4, (shape, R, variant)   # fp32 output of exact bf16 products
+        assert rel_err(S[r], db) <= 1e-4
+
+
+def test_reduce_sgd_writes_bf16_copy():
+    rng = np.random.default_rng(4)
+    n, R = 100003, 4
+    W = rng.uniform(-1, 1, n).astype(np.float32)
+    G = rng.standard_normal((R, n)).astype(np.float32)
+    dW, dG = capi.DeviceBuffer.from_numpy(W), capi.DeviceBuffer.from_numpy(G)
+    d16 = capi.DeviceBuffer(n * 2 + 16)
+    capi.check(capi.lib().mi_reduce_sgd_bf16_raw(dW.ptr, d16.ptr, dG.ptr, n, n, R, ctypes.c_float(0.01), None))
+    capi.check(capi.lib().mi_stream_sync(None))
+    want = oracle.reduce_sgd(W, G, 0.01)
+    got = dW.to_numpy((n,))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(d16.to_numpy((n,), np.uint16), to_bf16_bits(want))
+
+
+LR = 0.01
+STEP_CONFIGS = {
+    "square": ([256, 256, 256, 256], 128, 2),
+    "rect": ([256, 512, 128, 384], 128, 3),
+    "ragged": ([100, 72, 40, 24], 37, 2),
+}
+
+
+@pytest.mark.parametrize("name", list(STEP_CONFIGS))
+@pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, 0, capi.FLAG_PER_LAYER_UPDATE])
+def test_bf16_step_matches_fp32_oracle(name, flags):
+    nf, B, R = STEP_CONFIGS[name]
+    L = len(nf) - 1
+    X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed=31)
+    rng = np.random.default_rng(1)
+    bs = [(0.1 * rng.standard_normal(b.shape)).astype(np.float32) for b in bs]
+    h = capi.MlpHandle(nf, B, R, dtype=capi.MI_BF16, flags=flags)
+    for l in range(L):
+        h.set_weights(l, Ws[l], bs[l])
+    h.set_input(X)
+    h.set_dy(dY)
+    for _ in range(2 if flags == 0 else 1):   # with graphs: the second call is the replay
+        h.snapshot_weights() if _ == 0 else h.restore_weights()
+        h.step(LR)
+    h.sync()
+    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR)
+    acts = [h.activation(l) for l in range(L + 1)]
+    for l in range(L + 1):
+        assert rel_err(acts[l], ref.acts[l]) <= BF16_TOL, f"activation {l}"
+    # The ReLU mask [A > 0] is discontinuous: about one activation in a hundred lies closer to
+    # zero than the bf16 forward error, and each such flip changes a gradient entry by its full
+    # size.  The backward pass is therefore compared with the fp32 oracle evaluated on the
+    # device's own (bf16) activations, i.e. with identical masks.
+    flipped = sum(int(np.count_nonzero((acts[l] > 0) != (ref.acts[l] > 0))) for l in range(1, L))
+    total = sum(acts[l].size for l in range(1, L))
+    assert flipped <= 0.03 * total, f"{flipped} of {total} masks differ"
+    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR, given_acts=acts)
+    assert rel_err(h.dx(), ref.dX) <= BF16_TOL
+    for l in range(L):
+        for r in range(R):
+            assert rel_err(h.wgrad_of(l, r), ref.dW[r][l]) <= BF16_TOL, (l, r)
+            assert rel_err(h.bgrad_of(l, r), ref.db[r][l]) <= BF16_TOL, (l, r)
+        assert rel_err(h.weight(l), ref.W_new[l]) <= BF16_TOL
+        assert rel_err(h.bias(l), ref.b_new[l]) <= BF16_TOL
+    h.close()
+
+
+def test_bf16_master_weights_stay_fp32():
+    """The update is applied to the fp32 master copy: a step whose update is far below bf16
+    resolution still changes the weights."""
+    nf, B, R = [128, 128], 64, 1
+    X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed=2)
+    h = capi.MlpHandle(nf, B, R, dtype=capi.MI_BF16, flags=capi.FLAG_NO_GRAPH)
+    h.set_weights(0, Ws[0], bs[0])
+    h.set_input(X)
+    h.set_dy(dY)
+    h.step(1e-7)
+    h.sync()
+    W1 = h.weight(0)
+    assert not np.array_equal(W1, Ws[0])
+    assert np.abs(W1 - Ws[0]).max() < 1e-4
+    h.close()
