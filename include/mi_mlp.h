@@ -215,6 +215,10 @@ int mi_mlp_get_bias(mi_mlp* h, int l, float* dst);
 int mi_mlp_get_wgrad(mi_mlp* h, int l, int r, float* dst, int ld);
 int mi_mlp_get_bgrad(mi_mlp* h, int l, int r, float* dst);
 int mi_mlp_get_dx(mi_mlp* h, float* dst, int ld);
+/* Gradient with respect to the pre-activation output of layer l, [R*B x N_{l+1}]: the uploaded dY
+ * for l = L-1, otherwise what mi_fc_dgrad(l+1) produced.  The two gradient buffers alternate, so
+ * the value is only meaningful between mi_fc_dgrad(l+1) and mi_fc_dgrad(l-1). */
+int mi_mlp_get_dz(mi_mlp* h, int l, float* dst, int ld);
 
 /* Device-side copy of all weights and biases (snapshot) and its inverse (restore), both
  * asynchronous on the handle's stream.  A benchmark loop restores before every step so that the

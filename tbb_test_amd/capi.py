@@ -73,6 +73,7 @@ SIGNATURES = {
     "mi_mlp_get_wgrad": [c_void_p, c_int, c_int, c_void_p, c_int],
     "mi_mlp_get_bgrad": [c_void_p, c_int, c_int, c_void_p],
     "mi_mlp_get_dx": [c_void_p, c_void_p, c_int],
+    "mi_mlp_get_dz": [c_void_p, c_int, c_void_p, c_int],
     "mi_mlp_snapshot_weights": [c_void_p],
     "mi_mlp_restore_weights": [c_void_p],
     "mi_mlp_param_count": [c_void_p, POINTER(c_size_t), POINTER(c_size_t)],
@@ -227,6 +228,7 @@ class MlpHandle:
     def wgrad_of(self, l, r): return self._get(lib().mi_mlp_get_wgrad, (self.nf[l + 1], self.nf[l]), l, r)
     def bgrad_of(self, l, r): return self._get(lib().mi_mlp_get_bgrad, (self.nf[l + 1],), l, r)
     def dx(self): return self._get(lib().mi_mlp_get_dx, (self.MB, self.nf[0]))
+    def dz(self, l): return self._get(lib().mi_mlp_get_dz, (self.MB, self.nf[l + 1]), l)
 
     def snapshot_weights(self): check(lib().mi_mlp_snapshot_weights(self._h))
     def restore_weights(self): check(lib().mi_mlp_restore_weights(self._h))

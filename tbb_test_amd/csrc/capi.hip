@@ -845,6 +845,11 @@ int mi_mlp_restore_weights(mi_mlp* h) {
   return MI_OK;
 }
 
+int mi_mlp_get_dz(mi_mlp* h, int l, float* dst, int ld) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  return download_matrix(h, dst, dz_of_layer(h, l), h->MB, h->nf[l + 1], ld, h->dtype == MI_BF16);
+}
+
 int mi_mlp_param_count(mi_mlp* h, size_t* params, size_t* replica_stride) {
   if (int rc = check_handle(h)) return rc;
   if (params) *params = h->P;
