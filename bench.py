@@ -6,7 +6,8 @@
 A "step" is one pass of the whole hot path over one batch of seeded synthetic input: L forward
 GEMMs, L weight-gradient GEMMs (R replicas each), L bias gradients, L input-gradient GEMMs and
 the R-way gradient reduce with the SGD update.  Inputs and weights are resident in HBM before
-the timed region starts.  Every timed step starts from the initial weights (a device-to-device
+the timed region starts.  Default schedule: the weight-gradient GEMMs and the per-layer reduce+SGD
+launches trail the chain of input-gradient GEMMs on a second stream.  Every timed step starts from the initial weights (a device-to-device
 restore that is inside the timed region), so that values stay finite however many sum-reduced
 SGD steps are run.
 
@@ -15,7 +16,9 @@ Prints one JSON line:
                  3 * 2 * (R*B) * sum_l N_l*N_{l+1}   (mlp_omp.cc:492,584,675)
   ms_per_step    wall clock of the timed loop / K
   roofline       the GEMM kernels (the dominant kernels): FLOP per launch / average launch
-                 duration from HIP events on the launching stream, against the fp32 MFMA peak
+                 duration from HIP events on the launching stream, against the fp32 MFMA peak.
+                 Taken in a second pass over the same K steps in which every kernel runs alone
+                 (one stream, one update launch): overlapping kernels cannot be timed individually
   roofline_reduce  the reduce+SGD kernel: (R+2)*4*P bytes / its launch duration, against HBM peak
   cpu_baseline   the CPU restatement of the reference's mlp_omp timed on this host's cores
 """
@@ -65,7 +68,10 @@ def main():
     ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
     ap.add_argument("--lr", type=float, default=0.01)
     ap.add_argument("--seed", type=int, default=1)
-    ap.add_argument("--overlap", action="store_true", help="per-layer update on a second stream")
+    ap.add_argument("--flat-update", action="store_true",
+                    help="one update launch at the end of the step instead of per-layer updates on the second stream")
+    ap.add_argument("--variants", default="", help="tuning: forced GEMM tile variants 'nt,nn,tn'")
+    ap.add_argument("--serial-backward", action="store_true", help="whole backward pass on one stream")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg (0 = skip)")
     args = ap.parse_args()
 
@@ -83,8 +89,11 @@ def main():
     info = capi.device_info()
 
     X, Ws, dY = hostlib.init_problem(nf, B, R, args.seed)
-    flags = capi.FLAG_PER_LAYER_UPDATE if args.overlap else 0
+    flags = (0 if args.flat_update else capi.FLAG_PER_LAYER_UPDATE) | (capi.FLAG_SERIAL_BACKWARD if args.serial_backward else 0)
     h = capi.MlpHandle(nf, B, R, dtype=capi.MI_BF16 if dtype == "bf16" else capi.MI_F32, flags=flags)
+    if args.variants:
+        for kind, v in enumerate(int(x) for x in args.variants.split(",")):
+            capi.check(capi.lib().mi_set_gemm_variant(kind, v))
     for l in range(layers):
         h.set_weights(l, Ws[l], None)
     h.set_input(X)
@@ -134,10 +143,10 @@ def main():
 
     upd_launches = int(cnt[3].sum())
     upd_ms = float(ms[3].sum()) / upd_launches
-    # one launch covers all layers unless the per-layer schedule is on
-    upd_bytes = (R + 2) * 4.0 * params * (1 if not args.overlap else 1.0 / layers)
+    # the event-timed pass always runs the update as one launch over all layers
+    upd_bytes = (R + 2) * 4.0 * params
     if dtype == "bf16":
-        upd_bytes += 2.0 * params * (1 if not args.overlap else 1.0 / layers)
+        upd_bytes += 2.0 * params
     upd_gbps = upd_bytes / (upd_ms * 1e-3) / 1e9
 
     peak = PEAK_TFLOPS[dtype]
@@ -156,7 +165,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.config}: {layers} FC layers of width {width}, ReLU between layers, "
                                f"batch {B} per replica x {R} replicas, lr {args.lr}, seed {args.seed}",
-                   "schedule": "per-layer update on a second stream" if args.overlap else "one update launch",
+                   "schedule": ("serial backward" if args.serial_backward else "weight-gradient GEMMs on a second stream")
+                               + (", one update launch" if args.flat_update else ", per-layer update on the second stream"),
                    "device": info["name"], "num_cus": info["num_cus"]},
         "gemm_flop_per_step": gemm_flop_step,
         "phase_ms_per_step": {k: round(v, 4) for k, v in per_phase.items()},
@@ -166,13 +176,12 @@ def main():
         "roofline": {"kernel": "gemm_f32_mfma (nt, nn, tn)" if dtype == "f32" else "gemm_bf16_mfma",
                      "bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(gemm_tflops / peak, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get("gemm") if not args.overlap else None,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get("gemm"),
                      "flop_per_launch": flop_per_gemm, "avg_launch_us": round(gemm_avg_ms * 1e3, 2),
                      "launches": gemm_launches},
         "roofline_reduce": {"kernel": "reduce_sgd_vec4", "bound": "hbm", "achieved": round(upd_gbps, 1),
                             "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(upd_gbps / PEAK_HBM_GBPS, 4),
-                            "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get("reduce")
-                            if not args.overlap else None,
+                            "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get("reduce"),
                             "bytes_per_launch": upd_bytes, "avg_launch_us": round(upd_ms * 1e3, 2)},
     }
     if args.cpu_seconds > 0:

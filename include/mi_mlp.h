@@ -50,6 +50,10 @@ typedef enum mi_dtype {
                                     mlp_omp.cc:601-615,692-723 -- instead of one launch over all
                                     layers at the end of the step */
 
+#define MI_FLAG_SERIAL_BACKWARD 0x8u /* keep the whole backward pass on one stream; default: the
+                                    weight-gradient GEMMs run on a second stream next to the chain
+                                    of input-gradient GEMMs (they are independent per layer) */
+
 /* Timing slots, same names and order as the reference's enum Breakdown
  * (mlp_bench_common.h:12-20). */
 enum {
@@ -235,6 +239,8 @@ int mi_mlp_param_count(mi_mlp* h, size_t* params, size_t* replica_stride);
  * Per-phase device timing with HIP events on the handle's stream (the role of sum_times /
  * dsecnd() in mlp_omp.cc:490-508,582-600,673-691,161-168).  While enabled, every kernel of
  * mi_mlp_step and of the per-operation entry points is bracketed by an event pair.
+ * While timing is enabled the step runs serially on one stream with a single update launch,
+ * whatever the scheduling flags say, because overlapping kernels cannot be timed individually.
  * mi_mlp_get_timings synchronises and writes accumulated milliseconds as
  * ms[breakdown * L + layer]; the single all-layer reduce launch is booked under
  * MI_WGT_UPDATE, layer 0.  launches[] (same indexing, may be NULL) receives launch counts.

@@ -12,7 +12,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
 MI_F32, MI_BF16 = 0, 1
-FLAG_RELU_LAST, FLAG_NO_GRAPH, FLAG_PER_LAYER_UPDATE = 1, 2, 4
+FLAG_RELU_LAST, FLAG_NO_GRAPH, FLAG_PER_LAYER_UPDATE, FLAG_SERIAL_BACKWARD = 1, 2, 4, 8
 BREAKDOWN_NAMES = ("fwd", "wgt_grad", "bwd", "wgt_update", "wgt_update_reduce_scatter", "wgt_update_allgather")
 NUM_BREAKDOWNS = len(BREAKDOWN_NAMES)
 

@@ -74,13 +74,14 @@ struct mi_mlp {
   uint16_t* dzT = nullptr;       // bf16 only: per-replica transposed gradient [R][max N x B]
   std::vector<void*> acts;    // L+1 buffers [MB x nf[l]], fp32 or bf16
   void* dy = nullptr;         // upstream gradient [MB x nf[L]]
-  void* dz[2] = {nullptr, nullptr};  // gradient ping-pong [MB x max width]
+  void* dz[3] = {nullptr, nullptr, nullptr};  // gradient rotation [MB x max width]: dZ_l lives in dz[l % 3]
   void* dx = nullptr;         // gradient w.r.t. the input [MB x nf[0]]
   float* staging = nullptr;   // fp32 bounce buffer for bf16 uploads/downloads [MB x max width] or one W
   size_t staging_elems = 0;
   hipStream_t stream = nullptr, stream2 = nullptr;
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
-  std::vector<hipEvent_t> ev_layer;  // per-layer "input-gradient GEMM done" (overlapped update)
+  std::vector<hipEvent_t> ev_layer;  // per layer: input-gradient GEMM of layer l done (dZ_{l-1} ready, W_l free)
+  std::vector<hipEvent_t> ev_wgrad;  // per layer: weight-gradient GEMM of layer l done (dZ_l free)
 
   // timing
   bool timing = false;
@@ -167,7 +168,7 @@ struct TimedScope {
 const void* dz_of_layer(mi_mlp* h, int l) {
   // gradient w.r.t. the pre-activation output of layer l
   if (l == h->L - 1 && !(h->flags & MI_FLAG_RELU_LAST)) return h->dy;
-  return h->dz[l & 1];
+  return h->dz[l % 3];
 }
 
 int op_forward(mi_mlp* h, int l, hipStream_t s) {
@@ -233,7 +234,7 @@ int op_bgrad(mi_mlp* h, int l, hipStream_t s) {
 int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
   TimedScope ts(h, s, MI_BWD, l);
   if (ts.status) return ts.status;
-  void* out = (l == 0) ? h->dx : h->dz[(l - 1) & 1];
+  void* out = (l == 0) ? h->dx : h->dz[(l - 1) % 3];
   const void* mask = (l == 0) ? nullptr : h->acts[l];
   hipError_t e;
   if (h->dtype == MI_F32) {
@@ -286,38 +287,63 @@ int op_last_mask(mi_mlp* h, hipStream_t s) {
   const size_t n = (size_t)h->MB * h->nf[h->L];
   size_t blocks = (n + 255) / 256;
   if (blocks > 4096) blocks = 4096;
-  hipLaunchKernelGGL(mask_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float*)h->dz[(h->L - 1) & 1],
+  hipLaunchKernelGGL(mask_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float*)h->dz[(h->L - 1) % 3],
                      (const float*)h->dy, (const float*)h->acts[h->L], n);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e, "mask launch");
   return MI_OK;
 }
 
-// Enqueues one whole step.  With MI_FLAG_PER_LAYER_UPDATE the update of layer l runs on the second
-// stream as soon as layer l's input-gradient GEMM (the last reader of W_l) has finished, and the
-// main stream waits for all updates at the end.
+// Enqueues one whole step.
+//
+// Backward runs on two streams: the input-gradient GEMMs form the dependent chain on the main
+// stream, the weight-gradient GEMMs (which nothing in the backward pass depends on) trail them on
+// the second stream.  The two kinds are independent per layer, so the workgroups of one kernel move
+// onto CUs as the other kernel's workgroups drain, which hides the prologue and epilogue that a
+// chain of dependent one-tile-per-CU launches cannot hide.  dZ_l rotates through three buffers so
+// that dgrad(l-1) may overwrite nothing wgrad(l) still reads; dgrad(l) additionally waits for
+// wgrad(l+2), the last reader of the buffer it writes.  MI_FLAG_SERIAL_BACKWARD keeps everything on
+// one stream.  With MI_FLAG_PER_LAYER_UPDATE the update of layer l follows wgrad(l) on the second
+// stream as soon as dgrad(l), the last reader of W_l, is done; otherwise one update over all
+// layers closes the step.
 int enqueue_step(mi_mlp* h, float lr) {
   hipStream_t s = h->stream;
   int rc;
   for (int l = 0; l < h->L; ++l)
     if ((rc = op_forward(h, l, s))) return rc;
   if ((rc = op_last_mask(h, s))) return rc;
-  const bool overlap = (h->flags & MI_FLAG_PER_LAYER_UPDATE) != 0;
+  // While per-kernel event timing is on, everything runs back to back on one stream with one
+  // update launch: durations of kernels that overlap cannot be attributed to a kernel.
+  const bool per_layer = (h->flags & MI_FLAG_PER_LAYER_UPDATE) != 0 && !h->timing;
+  const bool dual = !(h->flags & MI_FLAG_SERIAL_BACKWARD) && !h->timing;
+  hipStream_t s2 = dual ? h->stream2 : s;
+  if (dual) {  // fork: dZ_{L-1} and all activations are ready
+    MI_HIP(hipEventRecord(h->ev_fork, s));
+    MI_HIP(hipStreamWaitEvent(s2, h->ev_fork, 0));
+  }
   for (int l = h->L - 1; l >= 0; --l) {
-    if ((rc = op_wgrad(h, l, s, true))) return rc;
+    if ((rc = op_wgrad(h, l, s2, true))) return rc;
+    if (dual) {
+      MI_HIP(hipEventRecord(h->ev_wgrad[l], s2));
+      if (l + 2 <= h->L - 1) MI_HIP(hipStreamWaitEvent(s, h->ev_wgrad[l + 2], 0));
+    }
     if ((rc = op_dgrad(h, l, s))) return rc;
-    if (overlap) {
+    if (dual || per_layer) {
       MI_HIP(hipEventRecord(h->ev_layer[l], s));
-      MI_HIP(hipStreamWaitEvent(h->stream2, h->ev_layer[l], 0));
-      if ((rc = op_update(h, l, lr, h->stream2))) return rc;
+      if (s2 != s) MI_HIP(hipStreamWaitEvent(s2, h->ev_layer[l], 0));  // wgrad(l-1) needs dZ_{l-1}; update(l) needs W_l free
+    }
+    if (per_layer) {
+      hipStream_t su = dual ? s2 : h->stream2;
+      if (!dual) MI_HIP(hipStreamWaitEvent(su, h->ev_layer[l], 0));
+      if ((rc = op_update(h, l, lr, su))) return rc;
     }
   }
-  if (overlap) {
+  if (dual || per_layer) {
     MI_HIP(hipEventRecord(h->ev_join, h->stream2));
     MI_HIP(hipStreamWaitEvent(s, h->ev_join, 0));
-  } else {
-    if ((rc = op_update(h, -1, lr, s))) return rc;
   }
+  if (!per_layer)
+    if ((rc = op_update(h, -1, lr, s))) return rc;
   return MI_OK;
 }
 
@@ -633,19 +659,21 @@ int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_repli
   h->acts.assign(L + 1, nullptr);
   for (int l = 0; l <= L; ++l) alloc(&h->acts[l], (size_t)h->MB * h->nf[l] * es);
   alloc(&h->dy, (size_t)h->MB * h->nf[L] * es);
-  alloc(&h->dz[0], (size_t)h->MB * h->maxw() * es);
-  alloc(&h->dz[1], (size_t)h->MB * h->maxw() * es);
+  for (int i = 0; i < 3; ++i) alloc(&h->dz[i], (size_t)h->MB * h->maxw() * es);
   alloc(&h->dx, (size_t)h->MB * h->nf[0] * es);
   if (rc == MI_OK && hipDeviceSynchronize() != hipSuccess) rc = fail(MI_ERR_HIP, "hipDeviceSynchronize failed");
   if (rc == MI_OK && hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking) != hipSuccess)
     rc = fail(MI_ERR_HIP, "hipStreamCreate failed");
-  if (rc == MI_OK && (flags & MI_FLAG_PER_LAYER_UPDATE)) {
+  if (rc == MI_OK) {
     if (hipStreamCreateWithFlags(&h->stream2, hipStreamNonBlocking) != hipSuccess ||
-        hipEventCreateWithFlags(&h->ev_join, hipEventDisableTiming) != hipSuccess)
+        hipEventCreateWithFlags(&h->ev_join, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&h->ev_fork, hipEventDisableTiming) != hipSuccess)
       rc = fail(MI_ERR_HIP, "second stream setup failed");
     h->ev_layer.assign(L, nullptr);
+    h->ev_wgrad.assign(L, nullptr);
     for (int l = 0; l < L && rc == MI_OK; ++l)
-      if (hipEventCreateWithFlags(&h->ev_layer[l], hipEventDisableTiming) != hipSuccess)
+      if (hipEventCreateWithFlags(&h->ev_layer[l], hipEventDisableTiming) != hipSuccess ||
+          hipEventCreateWithFlags(&h->ev_wgrad[l], hipEventDisableTiming) != hipSuccess)
         rc = fail(MI_ERR_HIP, "hipEventCreate failed");
   }
   if (rc != MI_OK) {
@@ -670,6 +698,8 @@ int mi_mlp_destroy(mi_mlp* h) {
   for (auto e : h->free_events) (void)hipEventDestroy(e);
   for (auto e : h->ev_layer)
     if (e) (void)hipEventDestroy(e);
+  for (auto e : h->ev_wgrad)
+    if (e) (void)hipEventDestroy(e);
   if (h->ev_join) (void)hipEventDestroy(h->ev_join);
   if (h->ev_fork) (void)hipEventDestroy(h->ev_fork);
   (void)hipFree(h->params);
@@ -683,8 +713,7 @@ int mi_mlp_destroy(mi_mlp* h) {
   (void)hipFree(h->dzT);
   for (void* a : h->acts) (void)hipFree(a);
   (void)hipFree(h->dy);
-  (void)hipFree(h->dz[0]);
-  (void)hipFree(h->dz[1]);
+  for (int i = 0; i < 3; ++i) (void)hipFree(h->dz[i]);
   (void)hipFree(h->dx);
   (void)hipFree(h->staging);
   if (h->stream) (void)hipStreamDestroy(h->stream);

@@ -16,8 +16,8 @@
 // Structure: as the fp32 kernel -- three LDS buffers, tile t+1 written to LDS at the top of step
 // t, loads of tile t+2 issued right after, one LDS-only barrier in the middle of the step,
 // operand fragments of the next 16-wide K chunk fetched while the current chunk is multiplied.
-// Tiles are stored [row][BK + 8] (16-byte pad per row); a lane fetches its 8 k values of one
-// 32 x 32 block with one 16-byte LDS read.
+// Tiles are stored [row][BK] with the 16-byte chunks of a row XOR-swizzled (no padding, no bank
+// conflicts); a lane fetches its 8 k values of one 32 x 32 block with one 16-byte LDS read.
 #include <hip/hip_runtime.h>
 
 #include "kernels.h"
@@ -60,12 +60,46 @@ __device__ __forceinline__ void lds_barrier_h() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int EPI>
+// Maps the flat workgroup index to a C tile.  Workgroups are handed to the 8 XCDs round-robin
+// (id % 8), each XCD has a private 4 MB L2, and about 32 workgroups (one per CU) of an XCD run at
+// the same time.
+//   * Large grids (tile counts divisible as needed): the grid is cut into super-tiles of 4 x 8
+//     tiles; XCD x owns super-tiles x, x+8, ... and walks each row by row, so the 32 tiles it
+//     runs together share 4 A panels and 8 B panels -- 12 panel slices per K step from the
+//     fabric instead of the 33 a single tile row needs.
+//   * Otherwise, if the tile count is a multiple of 8: XCD x gets the contiguous range
+//     [x*T/8, (x+1)*T/8) of the row-major order (tiles of one row share their A panel).
+//   * Otherwise the identity.
+__device__ __forceinline__ void tile_of_workgroup(int id, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  if ((tiles_m & 3) == 0 && (tiles_n & 7) == 0 && (total & 255) == 0) {
+    const int xcd = id & 7, j = id >> 3;
+    const int super = (j >> 5) * 8 + xcd, within = j & 31;
+    const int super_cols = tiles_n >> 3;
+    tm = (super / super_cols) * 4 + (within >> 3);
+    tn = (super % super_cols) * 8 + (within & 7);
+    return;
+  }
+  if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+  tm = id / tiles_n;
+  tn = id - tm * tiles_n;
+}
+
+// PF = distance, in K steps, between issuing a tile's global loads and writing it to LDS.  A bf16
+// step is short (BK = 32 is two MFMA chunks, about 1000 cycles), so one step does not cover an
+// L2 hit; PF register sets rotate, one per in-flight tile.
+// STAGES = 2: two LDS buffers and the plain schedule (loads of tile t+1 at the top of step t,
+// written to LDS at its end, barrier at the step boundary) -- what fits when BK = 64 makes a
+// 256 x 256 tile 72 KB per buffer.  BK = 64 matters for bandwidth: a tile row is then one whole
+// 128-byte cache line, where BK = 32 touches half a line per row and step.
+template <int BM, int BN, int BK, int WM, int WN, int EPI, int PF = 1, int STAGES = 3>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
+  static_assert(PF >= 1 && PF <= 3, "prefetch distance");
+  static_assert(STAGES == 3 || (STAGES == 2 && PF == 1), "two buffers only with the plain schedule");
   constexpr int NT = WM * WN * 64;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr int STRIDE = BK + 8;                 // bf16 elements per LDS row
+  constexpr int STRIDE = BK;                     // bf16 elements per LDS row: no padding, chunks swizzled
   constexpr int A_ELEMS = BM * STRIDE, B_ELEMS = BN * STRIDE;
   constexpr int VPR = BK / 8;                    // 16-byte vectors per tile row
   constexpr int NVA = BM * VPR / NT, NVB = BN * VPR / NT;
@@ -76,18 +110,14 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
 
   extern __shared__ __attribute__((aligned(16))) u16 smem_h[];
   auto As = [&](int buf) { return smem_h + buf * A_ELEMS; };
-  auto Bs = [&](int buf) { return smem_h + 3 * A_ELEMS + buf * B_ELEMS; };
+  auto Bs = [&](int buf) { return smem_h + STAGES * A_ELEMS + buf * B_ELEMS; };
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hi = lane >> 5;
   const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
 
-  // XCD-aware tile order: XCD x (workgroup id % 8) gets a contiguous range of the row-major
-  // tile order, so tiles that share an A panel share an L2
-  int id = blockIdx.x;
-  const int total = p.tiles_m * p.tiles_n;
-  if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
-  const int tile_m = id / p.tiles_n, tile_n = id - tile_m * p.tiles_n;
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const u16* __restrict__ a_ptr = p.A + (size_t)blockIdx.z * p.batchA + (size_t)m0 * p.lda;
@@ -101,51 +131,85 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  u32x4 ra[NVA], rb[NVB];
-  auto fetch = [&]() {
+  u32x4 ra[PF][NVA], rb[PF][NVB];
+  auto fetch = [&](u32x4 (&sa)[NVA], u32x4 (&sb)[NVB]) {
 #pragma unroll
     for (int i = 0; i < NVA; ++i) {
       const int idx = tid + i * NT, row = idx / VPR, c = idx % VPR;
-      ra[i] = *reinterpret_cast<const u32x4*>(a_ptr + (size_t)row * p.lda + c * 8);
+      sa[i] = *reinterpret_cast<const u32x4*>(a_ptr + (size_t)row * p.lda + c * 8);
     }
 #pragma unroll
     for (int i = 0; i < NVB; ++i) {
       const int idx = tid + i * NT, row = idx / VPR, c = idx % VPR;
-      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (size_t)row * p.ldb + c * 8);
+      sb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (size_t)row * p.ldb + c * 8);
     }
     a_ptr += BK;
     b_ptr += BK;
   };
-  auto stash = [&](int buf) {
+  // LDS layout.  Rows are stored back to back; the 16-byte chunk c of row r sits at chunk
+  // position c ^ swz(r), swz(r) = (r / rows per 256 bytes) mod chunks per row.  The LDS has 64
+  // banks of 4 bytes and serves a 16-byte access 16 lanes at a time: 16 lanes reading the same
+  // chunk of 16 consecutive rows (the fragment read) and 16 lanes writing consecutive chunks (the
+  // tile store) both touch every bank exactly once.
+  constexpr int ROWS_PER_LINE = 256 / (BK * 2) > 0 ? 256 / (BK * 2) : 1;
+  auto swz = [](int row) { return (row / ROWS_PER_LINE) % VPR; };
+  auto stash = [&](int buf, const u32x4 (&sa)[NVA], const u32x4 (&sb)[NVB]) {
 #pragma unroll
     for (int i = 0; i < NVA; ++i) {
       const int idx = tid + i * NT, row = idx / VPR, c = idx % VPR;
-      *reinterpret_cast<u32x4*>(As(buf) + row * STRIDE + c * 8) = ra[i];
+      *reinterpret_cast<u32x4*>(As(buf) + row * STRIDE + (c ^ swz(row)) * 8) = sa[i];
     }
 #pragma unroll
     for (int i = 0; i < NVB; ++i) {
       const int idx = tid + i * NT, row = idx / VPR, c = idx % VPR;
-      *reinterpret_cast<u32x4*>(Bs(buf) + row * STRIDE + c * 8) = rb[i];
+      *reinterpret_cast<u32x4*>(Bs(buf) + row * STRIDE + (c ^ swz(row)) * 8) = sb[i];
     }
   };
   auto load_frags = [&](bf16x8 (&fa)[TM], bf16x8 (&fb)[TN], int buf, int kk) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
-      fa[i] = *reinterpret_cast<const bf16x8*>(As(buf) + (wm0 + i * 32 + l32) * STRIDE + kk * 16 + hi * 8);
+    for (int i = 0; i < TM; ++i) {
+      const int row = wm0 + i * 32 + l32;
+      fa[i] = *reinterpret_cast<const bf16x8*>(As(buf) + row * STRIDE + ((kk * 2 + hi) ^ swz(row)) * 8);
+    }
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-      fb[j] = *reinterpret_cast<const bf16x8*>(Bs(buf) + (wn0 + j * 32 + l32) * STRIDE + kk * 16 + hi * 8);
+    for (int j = 0; j < TN; ++j) {
+      const int row = wn0 + j * 32 + l32;
+      fb[j] = *reinterpret_cast<const bf16x8*>(Bs(buf) + row * STRIDE + ((kk * 2 + hi) ^ swz(row)) * 8);
+    }
   };
 
   const int nk = p.K / BK;
-  fetch();
-  stash(0);
-  if (nk > 1) fetch();
+  fetch(ra[0], rb[0]);
+  stash(0, ra[0], rb[0]);
+  if constexpr (STAGES == 2) {
+    __syncthreads();
+    for (int t = 0; t < nk; ++t) {
+      const int cur = t & 1;
+      if (t + 1 < nk) fetch(ra[0], rb[0]);
+#pragma unroll
+      for (int kk = 0; kk < CH; ++kk) {
+        bf16x8 fa[TM], fb[TN];
+        load_frags(fa, fb, cur, kk);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+      if (t + 1 < nk) stash(cur ^ 1, ra[0], rb[0]);
+      __syncthreads();
+    }
+  } else {
+  // tile j (j >= 1) travels through register set j % PF
+#pragma unroll
+  for (int j = 1; j <= PF; ++j)
+    if (j < nk) fetch(ra[j % PF], rb[j % PF]);
   lds_barrier_h();
   bf16x8 fa[2][TM], fb[2][TN];
   load_frags(fa[0], fb[0], 0, 0);
   int cur = 0;
-  for (int t = 0; t < nk; ++t) {
+  // one K step; `set` holds tile t+1 on entry and receives tile t+1+PF
+  auto step = [&](int t, u32x4 (&sa)[NVA], u32x4 (&sb)[NVB]) {
     const int nxt = cur == 2 ? 0 : cur + 1;
 #pragma unroll
     for (int kk = 0; kk < CH; ++kk) {
@@ -153,8 +217,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
       if (kk + 1 < CH) load_frags(fa[fn], fb[fn], cur, kk + 1);
       else if (t + 1 < nk) load_frags(fa[fn], fb[fn], nxt, 0);
       if (kk == 0) {
-        if (t + 1 < nk) stash(nxt);
-        if (t + 2 < nk) fetch();
+        if (t + 1 < nk) stash(nxt, sa, sb);
+        if (t + 1 + PF < nk) fetch(sa, sb);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -164,6 +228,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
       if (kk == CH - 2) lds_barrier_h();
     }
     cur = nxt;
+  };
+  for (int t = 0; t < nk; t += PF) {
+#pragma unroll
+    for (int u = 0; u < PF; ++u)
+      if (t + u < nk) step(t + u, ra[(u + 1) % PF], rb[(u + 1) % PF]);  // t is a multiple of PF
+  }
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------
@@ -220,10 +290,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_generic(HGemmArgs p) {
   (reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC)[(size_t)row * p.ldc + col] = f2bf(v);
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int EPI>
+template <int BM, int BN, int BK, int WM, int WN, int EPI, int PF = 1, int STAGES = 3>
 static hipError_t launch_h(HGemmArgs& p, int batch, hipStream_t s) {
-  constexpr size_t lds_bytes = 3 * (size_t)(BM + BN) * (BK + 8) * sizeof(u16);
-  auto kern = gemm_bf16_mfma<BM, BN, BK, WM, WN, EPI>;
+  constexpr size_t lds_bytes = STAGES * (size_t)(BM + BN) * BK * sizeof(u16);
+  static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB of LDS");
+  auto kern = gemm_bf16_mfma<BM, BN, BK, WM, WN, EPI, PF, STAGES>;
   static bool attr_set = false;
   if (lds_bytes > 64 * 1024 && !attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -245,9 +316,11 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
                       p.batchB % 8 == 0 && p.K > 0;
   auto fits = [&](int bm, int bn, int bk) { return vec_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0; };
   if (variant == 0) {
+    // 256 x 256 tiles with 8 wavefronts once they cover the CUs, else smaller tiles for more
+    // workgroups
     const long long t256 = (long long)(p.M / 256) * (p.N / 256) * batch;
-    if (fits(256, 256, 32) && t256 >= 256) variant = 1;
-    else if (fits(128, 128, 32)) variant = 3;
+    if (fits(256, 256, 32) && t256 >= 256) variant = 4;
+    else if (fits(128, 128, 32) && (long long)(p.M / 128) * (p.N / 128) * batch >= 128) variant = 3;
     else if (fits(64, 64, 32)) variant = 5;
     else variant = -1;
   }
@@ -258,6 +331,12 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     case 4: if (fits(256, 256, 32)) return launch_h<256, 256, 32, 2, 4, EPI>(p, batch, s); break;
     case 5: if (fits(64, 64, 32)) return launch_h<64, 64, 32, 2, 2, EPI>(p, batch, s); break;
     case 6: if (fits(128, 128, 64)) return launch_h<128, 128, 64, 2, 2, EPI>(p, batch, s); break;
+    case 7: if (fits(256, 256, 64)) return launch_h<256, 256, 64, 2, 2, EPI, 1, 2>(p, batch, s); break;
+    case 8: if (fits(256, 256, 32)) return launch_h<256, 256, 32, 2, 4, EPI, 2>(p, batch, s); break;
+    case 9: if (fits(256, 256, 64)) return launch_h<256, 256, 64, 2, 4, EPI, 1, 2>(p, batch, s); break;
+    case 10: if (fits(256, 128, 64)) return launch_h<256, 128, 64, 2, 2, EPI, 1, 3>(p, batch, s); break;
+    case 11: if (fits(256, 128, 64)) return launch_h<256, 128, 64, 2, 4, EPI, 1, 3>(p, batch, s); break;
+    case 12: if (fits(128, 256, 64)) return launch_h<128, 256, 64, 2, 4, EPI, 1, 3>(p, batch, s); break;
     default: break;
   }
   hipLaunchKernelGGL((gemm_bf16_generic<EPI>), dim3((p.N + 15) / 16, (p.M + 15) / 16, batch), dim3(256), 0, s, p);

@@ -58,12 +58,25 @@ struct GemmArgs {
 };
 
 // Maps the flat workgroup index to a C tile.  Workgroups are handed to the 8 XCDs round-robin
-// (id % 8) and each XCD has a private L2; giving XCD x the contiguous range
-// [x*T/8, (x+1)*T/8) of the row-major tile order keeps the tiles that share an A panel (same
-// tile row) on one L2.  Falls back to the identity when the tile count is not a multiple of 8.
+// (id % 8), each XCD has a private 4 MB L2, and about 32 workgroups (one per CU) of an XCD run at
+// the same time.
+//   * Large grids (tile counts divisible as needed): the grid is cut into super-tiles of 4 x 8
+//     tiles; XCD x owns super-tiles x, x+8, ... and walks each row by row, so the 32 tiles it
+//     runs together share 4 A panels and 8 B panels.
+//   * Otherwise, if the tile count is a multiple of 8: XCD x gets the contiguous range
+//     [x*T/8, (x+1)*T/8) of the row-major order (tiles of one row share their A panel).
+//   * Otherwise the identity.
 __device__ __forceinline__ void tile_of_block(const GemmArgs& p, int& tm, int& tn) {
   int id = blockIdx.x;
   const int total = p.tiles_m * p.tiles_n;
+  if ((p.tiles_m & 3) == 0 && (p.tiles_n & 7) == 0 && (total & 255) == 0 && total >= 512) {
+    const int xcd = id & 7, j = id >> 3;
+    const int super = (j >> 5) * 8 + xcd, within = j & 31;
+    const int super_cols = p.tiles_n >> 3;
+    tm = (super / super_cols) * 4 + (within >> 3);
+    tn = (super % super_cols) * 8 + (within & 7);
+    return;
+  }
   if ((total & 7) == 0) {
     const int per_xcd = total >> 3;
     id = (id & 7) * per_xcd + (id >> 3);

@@ -53,7 +53,9 @@ CONFIGS = {
 
 @pytest.mark.parametrize("name", list(CONFIGS))
 @pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, capi.FLAG_NO_GRAPH | capi.FLAG_RELU_LAST,
-                                   capi.FLAG_NO_GRAPH | capi.FLAG_PER_LAYER_UPDATE])
+                                   capi.FLAG_NO_GRAPH | capi.FLAG_PER_LAYER_UPDATE,
+                                   capi.FLAG_NO_GRAPH | capi.FLAG_SERIAL_BACKWARD,
+                                   capi.FLAG_SERIAL_BACKWARD | capi.FLAG_PER_LAYER_UPDATE, 0])
 def test_step_matches_oracle(name, flags):
     nf, B, R = CONFIGS[name]
     h, (X, Ws, bs, dY) = build(nf, B, R, seed=2024, flags=flags, bias_scale=0.1)
