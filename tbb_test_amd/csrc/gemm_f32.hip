@@ -53,6 +53,9 @@ struct GemmArgs {
   // fused column sums of the A operand (TN only): colsum[z*batchColsum + m] = sum_k A[k][m]
   float* colsum;
   long long batchColsum;
+  // GUARD kernels: which 16-byte vector accesses the alignment of pointers and leading dimensions
+  // allows (bit 0: A loads, bit 1: B loads, bit 2: C stores and mask loads)
+  int vec_flags;
   // tile rasterisation
   int tiles_m, tiles_n;
 };
@@ -116,6 +119,49 @@ __device__ __forceinline__ void load_tile(f32x4 (&v)[NV], const float* __restric
       const int k = idx / (ROWS / 4), c4 = idx % (ROWS / 4);
       v[i] = *reinterpret_cast<const f32x4*>(base + (size_t)k * ld + c4 * 4);
     }
+  }
+}
+
+// Same for a tile that may stick out of the matrix (GUARD kernels): `op` points at the operand,
+// the tile covers rows [row0, row0 + ROWS) of `rows_total` and k in [k0, k0 + BK) of K; whatever
+// lies outside is read as zero, so the MFMAs need no special cases.
+template <int ROWS, int BK, bool KMAJOR, int NT, int NV>
+__device__ __forceinline__ void load_tile_guard(f32x4 (&v)[NV], const float* __restrict__ op, int ld, int row0,
+                                                int rows_total, int k0, int K, int tid, bool vec) {
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int idx = tid + i * NT;
+    f32x4 t = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (KMAJOR) {
+      const int row = row0 + idx / (BK / 4), k = k0 + (idx % (BK / 4)) * 4;
+      if (row < rows_total && k < K) {
+        const float* src = op + (size_t)row * ld + k;
+        if (vec && k + 3 < K) {
+          t = *reinterpret_cast<const f32x4*>(src);
+        } else if (k + 3 < K) {
+          t[0] = src[0]; t[1] = src[1]; t[2] = src[2]; t[3] = src[3];
+        } else {
+          t[0] = src[0];
+          if (k + 1 < K) t[1] = src[1];
+          if (k + 2 < K) t[2] = src[2];
+        }
+      }
+    } else {
+      const int k = k0 + idx / (ROWS / 4), row = row0 + (idx % (ROWS / 4)) * 4;
+      if (k < K && row < rows_total) {
+        const float* src = op + (size_t)k * ld + row;
+        if (vec && row + 3 < rows_total) {
+          t = *reinterpret_cast<const f32x4*>(src);
+        } else if (row + 3 < rows_total) {
+          t[0] = src[0]; t[1] = src[1]; t[2] = src[2]; t[3] = src[3];
+        } else {
+          t[0] = src[0];
+          if (row + 1 < rows_total) t[1] = src[1];
+          if (row + 2 < rows_total) t[2] = src[2];
+        }
+      }
+    }
+    v[i] = t;
   }
 }
 
@@ -189,10 +235,15 @@ __device__ __forceinline__ void load_frag(float (&frag)[TB][4], const float* lds
 //      8-wide K chunk are always fetched from LDS while the current chunk is multiplied.
 //      PF (1 or 2) is the distance, in K steps, between issuing a tile's global loads and
 //      writing it to LDS; 2 covers an L2 miss without stalling the step that needs the data.
+//
+// GUARD = true: M, N and K need not be multiples of the tile; loads outside the matrices read zero
+// and the epilogue skips what lies outside C.  (Leading dimensions and base pointers must still be
+// 16-byte aligned; anything else goes to the any-shape kernel below.)
 template <int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM = false,
-          int STAGES = 2, int PF = 1>
+          int STAGES = 2, int PF = 1, bool GUARD = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
   static_assert(STAGES == 2 || STAGES == 3, "two or three LDS buffers");
+  static_assert(!GUARD || (STAGES == 3 && PF == 1), "the guarded loads are written for the 3-stage loop");
   static_assert(STAGES == 2 || (BK / 8) % 2 == 0, "the 3-stage loop alternates two fragment sets per chunk");
   static_assert(!COLSUM || (!A_KMAJOR && (WM * WN * 64) % BM == 0 && BK % ((WM * WN * 64) / BM) == 0),
                 "fused column sums need A stored [k][m] and a whole number of k slices");
@@ -245,7 +296,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
   float csum = 0.0f;
 
   f32x4 ra[NVA], rb[NVB];
-  const int nk = p.K / BK;
+  const int nk = GUARD ? (p.K + BK - 1) / BK : p.K / BK;
+  int kt = 0;  // index of the next K tile to request (GUARD loads address from scratch)
+  const float* __restrict__ a_op = p.A + (size_t)blockIdx.z * p.batchA;
+  const float* __restrict__ b_op = p.B + (size_t)blockIdx.z * p.batchB;
   auto mfma_chunk = [&](const float (&fa)[TM][4], const float (&fb)[TN][4]) {
 #pragma unroll
     for (int q = 0; q < 4; ++q)
@@ -261,8 +315,14 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
     for (int k = 0; k < CS_ROWS; ++k) csum += col[k * TA::kStride];
   };
 
-  load_tile<BM, BK, A_KMAJOR, NT, NVA>(ra, a_ptr, p.lda, tid);
-  load_tile<BN, BK, B_KMAJOR, NT, NVB>(rb, b_ptr, p.ldb, tid);
+  if constexpr (GUARD) {
+    load_tile_guard<BM, BK, A_KMAJOR, NT, NVA>(ra, a_op, p.lda, m0, p.M, 0, p.K, tid, p.vec_flags & 1);
+    load_tile_guard<BN, BK, B_KMAJOR, NT, NVB>(rb, b_op, p.ldb, n0, p.N, 0, p.K, tid, p.vec_flags & 2);
+    kt = 1;
+  } else {
+    load_tile<BM, BK, A_KMAJOR, NT, NVA>(ra, a_ptr, p.lda, tid);
+    load_tile<BN, BK, B_KMAJOR, NT, NVB>(rb, b_ptr, p.ldb, tid);
+  }
   store_tile<BM, BK, A_KMAJOR, NT, NVA>(As(0), ra, tid);
   store_tile<BN, BK, B_KMAJOR, NT, NVB>(Bs(0), rb, tid);
 
@@ -296,10 +356,16 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
     // tiles with an odd index travel through (ra2, rb2), even ones through (ra, rb).
     f32x4 ra2[PF == 2 ? NVA : 1], rb2[PF == 2 ? NVB : 1];
     auto fetch = [&](auto& sa, auto& sb) {
-      a_ptr += a_step;
-      b_ptr += b_step;
-      load_tile<BM, BK, A_KMAJOR, NT, NVA>(sa, a_ptr, p.lda, tid);
-      load_tile<BN, BK, B_KMAJOR, NT, NVB>(sb, b_ptr, p.ldb, tid);
+      if constexpr (GUARD) {
+        load_tile_guard<BM, BK, A_KMAJOR, NT, NVA>(sa, a_op, p.lda, m0, p.M, kt * BK, p.K, tid, p.vec_flags & 1);
+        load_tile_guard<BN, BK, B_KMAJOR, NT, NVB>(sb, b_op, p.ldb, n0, p.N, kt * BK, p.K, tid, p.vec_flags & 2);
+        ++kt;
+      } else {
+        a_ptr += a_step;
+        b_ptr += b_step;
+        load_tile<BM, BK, A_KMAJOR, NT, NVA>(sa, a_ptr, p.lda, tid);
+        load_tile<BN, BK, B_KMAJOR, NT, NVB>(sb, b_ptr, p.ldb, tid);
+      }
     };
     if constexpr (PF == 2) {
       if (nk > 1) fetch(ra2, rb2);
@@ -358,7 +424,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
       float total = smem[tid];
 #pragma unroll
       for (int sl = 1; sl < CS_SLICES; ++sl) total += smem[sl * BM + tid];
-      p.colsum[(size_t)blockIdx.z * p.batchColsum + m0 + tid] = total;
+      if (!GUARD || m0 + tid < p.M) p.colsum[(size_t)blockIdx.z * p.batchColsum + m0 + tid] = total;
     }
   }
 
@@ -370,9 +436,16 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
   constexpr int CSTEP = B_KMAJOR ? 32 : 1;
   const float* __restrict__ mask = p.mask;
 
+  // GUARD: element (row, column j of this lane) exists
+  auto col_ok = [&](int j) { return !GUARD || col0 + j * CSTEP < p.N; };
+  constexpr bool VEC_STORE = !B_KMAJOR && (TN == 2 || TN == 4);
+  // a vector access covers TN consecutive columns starting at col0; with GUARD it needs all of them
+  const bool vec_ok = VEC_STORE && (!GUARD || ((p.vec_flags & 4) && col0 + TN - 1 < p.N));
+
   float bias_v[TN];
 #pragma unroll
-  for (int j = 0; j < TN; ++j) bias_v[j] = (EPI == EPI_BIAS_RELU && p.bias) ? p.bias[col0 + j * CSTEP] : 0.0f;
+  for (int j = 0; j < TN; ++j)
+    bias_v[j] = (EPI == EPI_BIAS_RELU && p.bias && col_ok(j)) ? p.bias[col0 + j * CSTEP] : 0.0f;
 
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
@@ -386,22 +459,26 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
     if (EPI == EPI_MASK) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float* mrow = mask + (size_t)row_of(r) * p.ldmask + col0;
-        if (!B_KMAJOR && TN == 4) {
+        const int row = row_of(r);
+        const float* mrow = mask + (size_t)row * p.ldmask + col0;
+        const bool row_ok = !GUARD || row < p.M;
+        if (VEC_STORE && TN == 4 && vec_ok && row_ok) {
           const f32x4 t = *reinterpret_cast<const f32x4*>(mrow);
           mk[r][0] = t[0]; mk[r][1 % TN] = t[1]; mk[r][2 % TN] = t[2]; mk[r][3 % TN] = t[3];
-        } else if (!B_KMAJOR && TN == 2) {
+        } else if (VEC_STORE && TN == 2 && vec_ok && row_ok) {
           const f32x2 t = *reinterpret_cast<const f32x2*>(mrow);
           mk[r][0] = t[0]; mk[r][1 % TN] = t[1];
         } else {
 #pragma unroll
-          for (int j = 0; j < TN; ++j) mk[r][j] = mrow[j * CSTEP];
+          for (int j = 0; j < TN; ++j) mk[r][j] = (row_ok && col_ok(j)) ? mrow[j * CSTEP] : 0.0f;
         }
       }
     }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      float* crow = C + (size_t)row_of(r) * p.ldc + col0;
+      const int row = row_of(r);
+      if (GUARD && row >= p.M) continue;
+      float* crow = C + (size_t)row * p.ldc + col0;
       float v[TN];
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
@@ -413,15 +490,16 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
           if (!(mk[r][j] > 0.0f)) v[j] = 0.0f;
         }
       }
-      if (!B_KMAJOR && TN == 4) {
+      if (VEC_STORE && TN == 4 && vec_ok) {
         const f32x4 o = {v[0], v[1 % TN], v[2 % TN], v[3 % TN]};
         *reinterpret_cast<f32x4*>(crow) = o;
-      } else if (!B_KMAJOR && TN == 2) {
+      } else if (VEC_STORE && TN == 2 && vec_ok) {
         const f32x2 o = {v[0], v[1 % TN]};
         *reinterpret_cast<f32x2*>(crow) = o;
       } else {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) crow[j * CSTEP] = v[j];
+        for (int j = 0; j < TN; ++j)
+          if (col_ok(j)) crow[j * CSTEP] = v[j];
       }
     }
   }
@@ -493,12 +571,13 @@ __global__ __launch_bounds__(256) void gemm_f32_generic(GemmArgs p) {
 
 // ---- launch ------------------------------------------------------------------------------------
 
-template <int BM, int BN, int BK, int WM, int WN, bool AK, bool BKM, int EPI, bool COLSUM, int STAGES = 2, int PF = 1>
+template <int BM, int BN, int BK, int WM, int WN, bool AK, bool BKM, int EPI, bool COLSUM, int STAGES = 2, int PF = 1,
+          bool GUARD = false>
 static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
   using TA = TileShape<BM, BK, AK>;
   using TB = TileShape<BN, BK, BKM>;
   constexpr size_t lds_bytes = STAGES * (TA::kFloats + TB::kFloats) * sizeof(float);
-  auto kern = gemm_f32_mfma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES, PF>;
+  auto kern = gemm_f32_mfma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES, PF, GUARD>;
   static bool attr_set = false;  // opt in to more than 64 KiB of dynamic LDS once per kernel
   if (lds_bytes > 64 * 1024 && !attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -506,8 +585,8 @@ static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  p.tiles_m = p.M / BM;
-  p.tiles_n = p.N / BN;
+  p.tiles_m = GUARD ? (p.M + BM - 1) / BM : p.M / BM;
+  p.tiles_n = GUARD ? (p.N + BN - 1) / BN : p.N / BN;
   dim3 grid(p.tiles_m * p.tiles_n, 1, batch);
   hipLaunchKernelGGL(kern, grid, dim3(WM * WN * 64), lds_bytes, s, p);
   return hipGetLastError();
@@ -531,7 +610,11 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
   const bool vec_ok = aligned16(p.A) && aligned16(p.B) && aligned16(p.C) && p.lda % 4 == 0 &&
                       p.ldb % 4 == 0 && p.ldc % 4 == 0 && p.batchA % 4 == 0 && p.batchB % 4 == 0 &&
                       p.batchC % 4 == 0 && p.K > 0;
-  auto fits = [&](int bm, int bn, int bk) { return vec_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0; };
+  // vector reads of the mask need the same alignment as the stores to C
+  const bool mask_ok = EPI != EPI_MASK || (aligned16(p.mask) && p.ldmask % 4 == 0);
+  auto fits = [&](int bm, int bn, int bk) {
+    return vec_ok && mask_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0;
+  };
   if (variant == 0) {
     // Automatic choice.  One 128 x 128 tile per CU (or more) keeps the chip busy with the
     // 8-wavefront, 3-stage kernel; smaller problems fall back to 128 x 64 and 64 x 64 tiles to
@@ -543,10 +626,18 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
       variant = 11;
     } else if (fits(64, 64, 16)) {
       variant = 16;
+    } else if (p.K > 0) {
+      // ragged shape or unaligned storage: the guarded MFMA kernels, big tile if it fills the chip
+      const long long t128 = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * batch;
+      variant = t128 >= 192 ? 21 : 22;
     } else {
       variant = -1;
     }
   }
+  // what the guarded kernels may access with 16-byte vectors
+  p.vec_flags = ((aligned16(p.A) && p.lda % 4 == 0 && p.batchA % 4 == 0) ? 1 : 0) |
+                ((aligned16(p.B) && p.ldb % 4 == 0 && p.batchB % 4 == 0) ? 2 : 0) |
+                ((aligned16(p.C) && p.ldc % 4 == 0 && p.batchC % 4 == 0 && mask_ok) ? 4 : 0);
   switch (variant) {
     case 1: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
     case 2: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
@@ -568,6 +659,8 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
     case 18: if (fits(128, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI, COLSUM, 3, 2>(p, batch, s); } break;
     case 19: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3, 2>(p, batch, s); } break;
     case 20: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 2, AK, BKM, EPI, COLSUM, 3, 2>(p, batch, s); } break;
+    case 21: if (p.K > 0) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 3, 1, true>(p, batch, s); } break;
+    case 22: if (p.K > 0) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<64, 64, 16, 2, 2, AK, BKM, EPI, COLSUM, 3, 1, true>(p, batch, s); } break;
     default: break;
   }
   return launch_generic<AK, BKM, EPI>(p, batch, s);

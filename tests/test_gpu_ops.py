@@ -83,8 +83,10 @@ GEMM_SHAPES = [
     (128, 128, 32), (256, 128, 64), (128, 256, 96), (512, 512, 512), (384, 640, 160),
     (64, 64, 32), (192, 64, 64),
     (1, 1, 1), (5, 3, 7), (100, 130, 50), (129, 127, 33), (257, 64, 1000), (64, 1, 64), (1, 300, 17),
+    # ragged but 16-byte aligned storage: the guarded MFMA kernels
+    (132, 260, 100), (1000, 520, 200), (36, 4, 64), (300, 128, 36), (128, 300, 4),
 ]
-VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20]
+VARIANTS = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20, 21, 22]
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
