@@ -83,6 +83,8 @@ struct mi_mlp {
   std::vector<hipEvent_t> ev_layer;  // per layer: input-gradient GEMM of layer l done (dZ_{l-1} ready, W_l free)
   std::vector<hipEvent_t> ev_wgrad;  // per layer: weight-gradient GEMM of layer l done (dZ_l free)
 
+  bool corun = false;  // set while enqueue_step issues the two backward chains on two streams
+
   // timing
   bool timing = false;
   struct Pair { hipEvent_t a, b; int slot; };
@@ -196,7 +198,8 @@ int op_wgrad(mi_mlp* h, int l, hipStream_t s, bool with_bias) {
   if (h->dtype == MI_F32) {
     e = mi::sgemm_tn(h->R, h->nf[l + 1], h->nf[l], h->B, (const float*)dz_of_layer(h, l), h->nf[l + 1],
                      (const float*)h->acts[l], h->nf[l], const_cast<float*>(g0), h->nf[l], (long long)h->stride,
-                     with_bias ? h->grads + h->boff[l] : nullptr, (long long)h->stride, s, g_variant[2]);
+                     with_bias ? h->grads + h->boff[l] : nullptr, (long long)h->stride, s,
+                     g_variant[2] ? g_variant[2] : (h->corun ? 100 : 0));
   } else {
     // K-contiguous copies of both operands, per replica: A_l^T [N_l x B] and dZ_l^T [N_{l+1} x B]
     const int B = h->B, nin = h->nf[l], nout = h->nf[l + 1];
@@ -240,7 +243,7 @@ int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
   if (h->dtype == MI_F32) {
     e = mi::sgemm_nn(h->MB, h->nf[l], h->nf[l + 1], (const float*)dz_of_layer(h, l), h->nf[l + 1],
                      h->params + h->woff[l], h->nf[l], (float*)out, h->nf[l], (const float*)mask, h->nf[l], s,
-                     g_variant[1]);
+                     g_variant[1] ? g_variant[1] : (h->corun ? 100 : 0));
   } else {
     e = mi::hgemm_nt(1, h->MB, h->nf[l], h->nf[l + 1], (const uint16_t*)dz_of_layer(h, l), h->nf[l + 1], 0,
                      h->params16T + h->woff[l], h->nf[l + 1], 0, out, h->nf[l], 0, mask ? 2 : 3, nullptr, 0,
@@ -321,7 +324,19 @@ int enqueue_step(mi_mlp* h, float lr) {
     MI_HIP(hipEventRecord(h->ev_fork, s));
     MI_HIP(hipStreamWaitEvent(s2, h->ev_fork, 0));
   }
+  // The backward GEMMs of a layer are told when they run next to each other with about one tile
+  // per CU each (then the kernels with the small LDS footprint share CUs).  The hint follows the
+  // configured schedule, not the momentary one, so that the per-kernel timing pass measures the
+  // kernels the real step uses.
+  struct CorunScope {
+    mi_mlp* h;
+    explicit CorunScope(mi_mlp* h_) : h(h_) {}
+    ~CorunScope() { h->corun = false; }
+  } corun_scope(h);
+  const bool corun_cfg = !(h->flags & MI_FLAG_SERIAL_BACKWARD);
   for (int l = h->L - 1; l >= 0; --l) {
+    const long long wgrad_tiles = (long long)(h->nf[l + 1] / 128) * (h->nf[l] / 128) * h->R;
+    h->corun = corun_cfg && wgrad_tiles < 512;
     if ((rc = op_wgrad(h, l, s2, true))) return rc;
     if (dual) {
       MI_HIP(hipEventRecord(h->ev_wgrad[l], s2));

@@ -615,12 +615,22 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
   auto fits = [&](int bm, int bn, int bk) {
     return vec_ok && mask_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0;
   };
+  // variant 100 = automatic, and the caller runs another GEMM next to this one on a second stream:
+  // then the 61 KB kernel pays off from one tile per CU on, because workgroups of the two kernels
+  // share CUs.
+  const bool corun = variant == 100;
+  if (corun) variant = 0;
   if (variant == 0) {
-    // Automatic choice.  One 128 x 128 tile per CU (or more) keeps the chip busy with the
-    // 8-wavefront, 3-stage kernel; smaller problems fall back to 128 x 64 and 64 x 64 tiles to
-    // get enough workgroups.
+    // Automatic choice among the 8-wavefront, 3-stage kernels on 128 x 128 tiles.  With two or more
+    // tiles per CU take BK = 16: its three LDS buffers are 61 KB, so two workgroups share a CU and
+    // one's prologue, epilogue and barrier waits are covered by the other's MFMAs.  With about one
+    // tile per CU nothing can overlap, and BK = 32 (110 KB, one workgroup per CU, half as many
+    // barriers) is faster.  Smaller problems fall back to 128 x 64 and 64 x 64 tiles to get
+    // enough workgroups.
     const long long tiles128 = (long long)(p.M / 128) * (p.N / 128) * batch;
-    if (fits(128, 128, 32) && tiles128 >= 192) {
+    if (fits(128, 128, 32) && (tiles128 >= 512 || (corun && tiles128 >= 192))) {
+      variant = 10;
+    } else if (fits(128, 128, 32) && tiles128 >= 192) {
       variant = 8;
     } else if (fits(128, 64, 32) && tiles128 * 2 >= 192) {
       variant = 11;
