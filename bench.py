@@ -45,7 +45,8 @@ METRIC = "MLP fwd+bwd+reduce step ms & TFLOP/s on 1 MI355X; grad-reduce GB/s"
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark
 # (FETCH_SIZE scaled by 1.9986, WRITE_SIZE by 1.0, the factors a plain 33.6 MB device copy gives;
-# the runs are summarised under profiles/).  GEMM: mean over the forward, weight-gradient and
+# the runs are summarised under profiles/; the BK = 16 kernels the default schedule uses for the
+# backward GEMMs read the same panels as the BK = 32 kernels these were taken on).  GEMM: mean over the forward, weight-gradient and
 # input-gradient launches.  None = not measured for that configuration.
 MEASURED_TRAFFIC_BYTES = {
     "C2": {"gemm": (50.4e6 + 16.8e6 + 151.0e6 + 16.8e6 + 67.2e6 + 16.8e6) / 3, "reduce": 167.8e6 + 33.6e6},
