@@ -85,6 +85,42 @@ __device__ __forceinline__ void tile_of_workgroup(int id, int tiles_m, int tiles
   tn = id - tm * tiles_n;
 }
 
+// Writes a wavefront's TM x TN accumulator blocks (32 x 32 each) with the epilogue EPI.  Lane l,
+// register r of a block hold row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+template <int TM, int TN, int EPI>
+__device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[TM][TN], int row0, int colw, int l32,
+                                             int hi) {
+  const int col0 = colw + l32;
+  float bias_v[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) bias_v[j] = (EPI == EPH_BIAS_RELU && p.bias) ? p.bias[col0 + j * 32] : 0.0f;
+  float* __restrict__ cf = reinterpret_cast<float*>(p.C) + (size_t)blockIdx.z * p.batchC;
+  u16* __restrict__ ch = reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = row0 + i * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = col0 + j * 32;
+        float v = acc[i][j][r];
+        if (EPI == EPH_F32) {
+          cf[(size_t)row * p.ldc + col] = v;
+        } else {
+          if (EPI == EPH_BIAS_RELU) {
+            v += bias_v[j];
+            if (p.relu) v = v > 0.0f ? v : 0.0f;
+          } else if (EPI == EPH_MASK) {
+            if (!(bf2f(p.mask[(size_t)row * p.ldmask + col]) > 0.0f)) v = 0.0f;
+          }
+          ch[(size_t)row * p.ldc + col] = f2bf(v);
+        }
+      }
+    }
+  }
+}
+
 // PF = distance, in K steps, between issuing a tile's global loads and writing it to LDS.  A bf16
 // step is short (BK = 32 is two MFMA chunks, about 1000 cycles), so one step does not cover an
 // L2 hit; PF register sets rotate, one per in-flight tile.
@@ -236,36 +272,195 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
   }
   }
 
-  // ---- epilogue ---------------------------------------------------------------------------------
-  const int col0 = n0 + wn0 + l32;
-  float bias_v[TN];
+  store_tile_h<TM, TN, EPI>(p, acc, m0 + wm0, n0 + wn0, l32, hi);
+}
+
+// ---- the same GEMM with direct global -> LDS loads ------------------------------------------------
+// global_load_lds_dwordx4 moves 16 bytes per lane from global memory straight into the LDS: the
+// 64 lanes of one instruction fill 1 KB of consecutive LDS bytes starting at a wave-uniform base
+// (lane i lands at base + 16 i), while each lane names its own global address.  The tile never
+// passes through VGPRs, so the ds_write traffic of the register-staged kernel (which costs about
+// as much LDS time as the fragment reads and kept the MFMA pipe waiting) disappears.  The XOR
+// swizzle of the LDS layout is produced on the global side: the lane that fills chunk position
+// pc of row r fetches the row's logical chunk pc ^ swz(r).
+//
+// Ring of STAGES LDS buffers.  In the middle of step t every wave waits (vmcnt) until its own
+// loads of tile t+1 have landed, all waves meet at one barrier, and the loads of tile t+STAGES-1
+// are issued into the buffer that step t-1 read.  Loads therefore have STAGES-2 whole steps to
+// complete; the counter wait leaves the younger tiles in flight.
+//
+// The load is written as inline assembly on purpose.  The compiler models the corresponding builtin
+// as a FLAT access that may touch both memories and then turns every later LDS-counter wait into
+// lgkmcnt(0) while such a load is pending, which serialises the fragment reads with the MFMAs.
+// Written this way the compiler does not track the load at all; the kernel waits on vmcnt itself
+// (its own waits can only become longer through the extra loads in flight, never shorter, because
+// vmcnt retires in order).  m0 carries the wave-uniform LDS byte address.
+__device__ __forceinline__ void load_to_lds(const u16* src, unsigned lds_byte_addr) {
+  const unsigned lds_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr);
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory", "m0");
+}
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
+// expcnt 6:4, lgkmcnt 11:8; the other counters at their maximum = no wait).
+constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x70 | 0xf00; }
+
+// Barrier of the ring: no LDS-counter wait is attached (nothing was written with ds_write, and a
+// buffer is refilled only after the MFMAs that consumed its last fragments, i.e. after those reads
+// returned); the empty asm statements keep the compiler from moving LDS reads across it.
+__device__ __forceinline__ void ring_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int EPI, int STAGES>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
+  constexpr int NW = WM * WN;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int STRIDE = BK;
+  constexpr int A_ELEMS = BM * STRIDE, B_ELEMS = BN * STRIDE;
+  constexpr int VPR = BK / 8;        // 16-byte chunks per tile row
+  constexpr int RPI = 64 / VPR;      // tile rows one load instruction of a wave fills
+  constexpr int NIA = BM / (RPI * NW), NIB = BN / (RPI * NW);
+  constexpr int INSTR = NIA + NIB;   // load instructions per wave and tile
+  constexpr int CH = BK / 16;
+  static_assert(STAGES >= 2 && STAGES <= 5, "ring depth");
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0 && CH % 2 == 0, "tile shape");
+  static_assert(BM % (RPI * NW) == 0 && BN % (RPI * NW) == 0, "tile must divide over the waves");
+  static_assert(STAGES == 2 || (STAGES - 2) * INSTR <= 63, "vmcnt is a 6-bit counter");
+
+  extern __shared__ __attribute__((aligned(16))) u16 smem_h[];
+  auto As = [&](int buf) { return smem_h + buf * A_ELEMS; };
+  auto Bs = [&](int buf) { return smem_h + STAGES * A_ELEMS + buf * B_ELEMS; };
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hi = lane >> 5;
+  const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
+
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  constexpr int ROWS_PER_LINE = 256 / (BK * 2) > 0 ? 256 / (BK * 2) : 1;
+  auto swz = [](int row) { return (row / ROWS_PER_LINE) % VPR; };
+
+  // global source of this lane for each of its load instructions
+  const int lrow = lane / VPR, pc = lane % VPR;
+  const u16* ga[NIA];
+  const u16* gb[NIB];
 #pragma unroll
-  for (int j = 0; j < TN; ++j) bias_v[j] = (EPI == EPH_BIAS_RELU && p.bias) ? p.bias[col0 + j * 32] : 0.0f;
-  float* __restrict__ cf = reinterpret_cast<float*>(p.C) + (size_t)blockIdx.z * p.batchC;
-  u16* __restrict__ ch = reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC;
+  for (int j = 0; j < NIA; ++j) {
+    const int row = (j * NW + wave) * RPI + lrow;
+    ga[j] = p.A + (size_t)blockIdx.z * p.batchA + (size_t)(m0 + row) * p.lda + (pc ^ swz(row)) * 8;
+  }
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+  for (int j = 0; j < NIB; ++j) {
+    const int row = (j * NW + wave) * RPI + lrow;
+    gb[j] = p.B + (size_t)blockIdx.z * p.batchB + (size_t)(n0 + row) * p.ldb + (pc ^ swz(row)) * 8;
+  }
+  const unsigned lds_base = (unsigned)(size_t)((__attribute__((address_space(3))) const void*)smem_h);
+  auto issue = [&](int buf) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
+    for (int j = 0; j < NIA; ++j) {
+      load_to_lds(ga[j], lds_base + 2u * (unsigned)(buf * A_ELEMS + (j * NW + wave) * RPI * STRIDE));
+      ga[j] += BK;
+    }
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int col = col0 + j * 32;
-        float v = acc[i][j][r];
-        if (EPI == EPH_F32) {
-          cf[(size_t)row * p.ldc + col] = v;
-        } else {
-          if (EPI == EPH_BIAS_RELU) {
-            v += bias_v[j];
-            if (p.relu) v = v > 0.0f ? v : 0.0f;
-          } else if (EPI == EPH_MASK) {
-            if (!(bf2f(p.mask[(size_t)row * p.ldmask + col]) > 0.0f)) v = 0.0f;
-          }
-          ch[(size_t)row * p.ldc + col] = f2bf(v);
+    for (int j = 0; j < NIB; ++j) {
+      load_to_lds(gb[j], lds_base + 2u * (unsigned)(STAGES * A_ELEMS + buf * B_ELEMS + (j * NW + wave) * RPI * STRIDE));
+      gb[j] += BK;
+    }
+  };
+  auto load_frags = [&](bf16x8 (&fa)[TM], bf16x8 (&fb)[TN], int buf, int kk) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = wm0 + i * 32 + l32;
+      fa[i] = *reinterpret_cast<const bf16x8*>(As(buf) + row * STRIDE + ((kk * 2 + hi) ^ swz(row)) * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int row = wn0 + j * 32 + l32;
+      fb[j] = *reinterpret_cast<const bf16x8*>(Bs(buf) + row * STRIDE + ((kk * 2 + hi) ^ swz(row)) * 8);
+    }
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int nk = p.K / BK;
+  bf16x8 fa[2][TM], fb[2][TN];
+  auto multiply = [&](int fc) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[fc][i], fb[fc][j], acc[i][j], 0, 0, 0);
+  };
+  if constexpr (STAGES == 2) {
+    // Two buffers (what fits when BK = 64 makes a 256 x 256 tile 64 KB): the loads of tile t+1 are
+    // issued at the top of step t into the buffer step t-1 read and have the whole step to land;
+    // one barrier at the step boundary.  BK = 64 rows are whole 128-byte lines, which the load path
+    // moves markedly faster than the half lines of BK = 32.
+    if (nk > 0) issue(0);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    ring_barrier();
+    for (int t = 0; t < nk; ++t) {
+      const int cur = t & 1;
+      if (t + 1 < nk) issue(cur ^ 1);
+      load_frags(fa[0], fb[0], cur, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kk = 0; kk < CH; ++kk) {
+        const int fc = kk & 1, fn = fc ^ 1;
+        if (kk + 1 < CH) load_frags(fa[fn], fb[fn], cur, kk + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(fc);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+      ring_barrier();
+    }
+  } else {
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s)
+      if (s < nk) issue(s);
+    if (nk >= STAGES - 1) __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * INSTR));
+    else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    ring_barrier();
+
+    load_frags(fa[0], fb[0], 0, 0);
+    int cur = 0;
+    for (int t = 0; t < nk; ++t) {
+      const int nxt = cur + 1 == STAGES ? 0 : cur + 1;
+      const int fill = cur == 0 ? STAGES - 1 : cur - 1;
+#pragma unroll
+      for (int kk = 0; kk < CH; ++kk) {
+        const int fc = kk & 1, fn = fc ^ 1;
+        if (kk + 1 < CH) load_frags(fa[fn], fb[fn], cur, kk + 1);
+        else load_frags(fa[fn], fb[fn], nxt, 0);  // after the last tile: a harmless read of ring memory, keeps one code path
+        // the scheduler otherwise sinks these reads below the MFMAs they are meant to overlap
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(fc);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kk == CH - 2) {
+          // tiles t+1 .. t+STAGES-2 are in flight; tile t+1 must have landed
+          if (t + STAGES - 2 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * INSTR));
+          else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+          ring_barrier();
+          if (t + STAGES - 1 < nk) issue(fill);
         }
       }
+      cur = nxt;
     }
   }
+  store_tile_h<TM, TN, EPI>(p, acc, m0 + wm0, n0 + wn0, l32, hi);
 }
 
 // Any-shape fallback: one thread per output element, fp32 accumulation in k order.
@@ -308,6 +503,24 @@ static hipError_t launch_h(HGemmArgs& p, int batch, hipStream_t s) {
   return hipGetLastError();
 }
 
+template <int BM, int BN, int BK, int WM, int WN, int EPI, int STAGES>
+static hipError_t launch_dma(HGemmArgs& p, int batch, hipStream_t s) {
+  constexpr size_t lds_bytes = STAGES * (size_t)(BM + BN) * BK * sizeof(u16);
+  static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB of LDS");
+  auto kern = gemm_bf16_dma<BM, BN, BK, WM, WN, EPI, STAGES>;
+  static bool attr_set = false;
+  if (lds_bytes > 64 * 1024 && !attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  p.tiles_m = p.M / BM;
+  p.tiles_n = p.N / BN;
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
+  return hipGetLastError();
+}
+
 template <int EPI>
 static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant) {
   if (p.M <= 0 || p.N <= 0 || batch <= 0) return hipSuccess;
@@ -316,10 +529,11 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
                       p.batchB % 8 == 0 && p.K > 0;
   auto fits = [&](int bm, int bn, int bk) { return vec_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0; };
   if (variant == 0) {
-    // 256 x 256 tiles with 8 wavefronts once they cover the CUs, else smaller tiles for more
-    // workgroups
+    // 256 x 256 tiles with 8 wavefronts and direct-to-LDS loads once they cover the CUs (whole
+    // 128-byte lines per row when K allows BK = 64), else smaller tiles for more workgroups
     const long long t256 = (long long)(p.M / 256) * (p.N / 256) * batch;
-    if (fits(256, 256, 32) && t256 >= 256) variant = 4;
+    if (fits(256, 256, 64) && t256 >= 256) variant = 19;
+    else if (fits(256, 256, 32) && t256 >= 256) variant = 13;
     else if (fits(128, 128, 32) && (long long)(p.M / 128) * (p.N / 128) * batch >= 128) variant = 3;
     else if (fits(64, 64, 32)) variant = 5;
     else variant = -1;
@@ -337,6 +551,15 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     case 10: if (fits(256, 128, 64)) return launch_h<256, 128, 64, 2, 2, EPI, 1, 3>(p, batch, s); break;
     case 11: if (fits(256, 128, 64)) return launch_h<256, 128, 64, 2, 4, EPI, 1, 3>(p, batch, s); break;
     case 12: if (fits(128, 256, 64)) return launch_h<128, 256, 64, 2, 4, EPI, 1, 3>(p, batch, s); break;
+    case 13: if (fits(256, 256, 32)) return launch_dma<256, 256, 32, 2, 4, EPI, 4>(p, batch, s); break;
+    case 14: if (fits(256, 256, 32)) return launch_dma<256, 256, 32, 2, 4, EPI, 3>(p, batch, s); break;
+    case 15: if (fits(256, 256, 32)) return launch_dma<256, 256, 32, 2, 2, EPI, 4>(p, batch, s); break;
+    case 16: if (fits(256, 128, 64)) return launch_dma<256, 128, 64, 2, 4, EPI, 3>(p, batch, s); break;
+    case 17: if (fits(128, 128, 32)) return launch_dma<128, 128, 32, 2, 2, EPI, 4>(p, batch, s); break;
+    case 18: if (fits(128, 128, 64)) return launch_dma<128, 128, 64, 2, 2, EPI, 4>(p, batch, s); break;
+    case 19: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2>(p, batch, s); break;
+    case 20: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 4, 2, EPI, 2>(p, batch, s); break;
+    case 21: if (fits(256, 256, 32)) return launch_dma<256, 256, 32, 2, 4, EPI, 5>(p, batch, s); break;
     default: break;
   }
   hipLaunchKernelGGL((gemm_bf16_generic<EPI>), dim3((p.N + 15) / 16, (p.M + 15) / 16, batch), dim3(256), 0, s, p);
