@@ -249,6 +249,32 @@ int mi_mlp_enable_timing(mi_mlp* h, int on);
 int mi_mlp_reset_timings(mi_mlp* h);
 int mi_mlp_get_timings(mi_mlp* h, double* ms, long long* launches);
 
+/*
+ * Loss front-end: SquaredL2Distance + AveragedLoss per replica as in the Caffe2 harness
+ * (mlp_caffe2.py:221-239): loss_r = (1/B) sum_{i in replica r} 0.5 * |pred_i - label_i|^2, the
+ * total is the sum over replicas, and the upstream gradient is dY = (pred - label) / B.
+ * mi_mlp_set_labels uploads Y [R*B x N_L] (fp32 on the device for both dtypes) and switches the
+ * handle to "loss mode": every mi_mlp_step then derives dY from its own forward output.
+ * mi_mlp_set_dy switches back to a given dY.  mi_loss_backward is the per-operation entry point
+ * (after mi_fc_forward(L-1), before the backward calls).  mi_mlp_get_loss synchronises and
+ * returns the losses of the last step (either pointer may be NULL).
+ */
+int mi_mlp_set_labels(mi_mlp* h, const float* Y, int ld);
+int mi_loss_backward(mi_mlp* h);
+int mi_mlp_get_loss(mi_mlp* h, double* loss_per_replica, double* total);
+
+/*
+ * Runs one step (like mi_mlp_step, eagerly, on the configured two-stream schedule) with an event
+ * pair around every launch and writes the timeline to `path` in the format of the reference's
+ * trace.log (mlp_tbb.cc:85-104,1379-1392: a JSON array of begin/end records with ts in
+ * microseconds, loadable in a Chrome-trace viewer).  Names follow the reference's tasks
+ * (mlp_tbb.cc:176-178,325-327,840,982,1104): FC_<l>_0, FCWgtGradient_<l>_0, FCBwdGradient_<l>_0;
+ * the fused reduce + SGD launch of layer l is ReduceScatterAllGather_<l>_0 (_all_ when one launch
+ * covers every layer), the loss kernel L2Loss_0.  pid 0 is the GPU, tid 0 / 1 the main / second
+ * stream.  The step updates the weights like any other.
+ */
+int mi_mlp_trace_step(mi_mlp* h, float lr, const char* path);
+
 #ifdef __cplusplus
 }
 #endif

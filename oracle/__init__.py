@@ -34,7 +34,8 @@ def _load():
         lib.oracle_mlp_step.argtypes = [_ci, ctypes.POINTER(_ci), _ci, _ci, _ci, _ci, ctypes.c_float, _vp, _vp, _vp, _vp,
                                         _vp, _vp]
         lib.oracle_mlp_step.restype = _ci
-        for fn in (lib.oracle_fc_forward, lib.oracle_fc_wgrad, lib.oracle_fc_dgrad, lib.oracle_reduce_sgd):
+        lib.oracle_l2_loss.argtypes = [_ci, _ci, _ci, _vp, _ci, _vp, _ci, _vp, _ci, _vp]
+        for fn in (lib.oracle_fc_forward, lib.oracle_fc_wgrad, lib.oracle_fc_dgrad, lib.oracle_reduce_sgd, lib.oracle_l2_loss):
             fn.restype = None
         _lib = lib
     return _lib
@@ -98,6 +99,19 @@ def reduce_sgd(W, G, lr):
 
 class StepResult:
     pass
+
+
+def l2_loss(pred, label, R):
+    """SquaredL2Distance + AveragedLoss per replica and its gradient w.r.t. pred.
+    pred, label: [R*B, N].  Returns (dY [R*B, N] float32, loss_per_replica [R] float64)."""
+    pred, label = _c(pred), _c(label)
+    MB, N = pred.shape
+    assert label.shape == pred.shape and MB % R == 0
+    dY = np.empty_like(pred)
+    loss = np.zeros(R, dtype=np.float64)
+    lib = _load()
+    lib.oracle_l2_loss(R, MB // R, N, _p(pred), N, _p(label), N, _p(dY), N, loss.ctypes.data_as(ctypes.c_void_p))
+    return dY, loss
 
 
 def mlp_step(nf, B, R, X, dY, Ws, bs, lr, relu_last=False, given_acts=None):

@@ -95,6 +95,30 @@ void oracle_fc_dgrad(int M, int N, int K, const float* dZ, int lddz, const float
   }
 }
 
+/* Loss front-end of the Caffe2 harness (mlp_caffe2.py:221-239): per replica
+ *   dist_i = 0.5 * sum_j (label[i][j] - pred[i][j])^2      (SquaredL2Distance, one value per row)
+ *   loss_r = (1/B) * sum_{i in replica r} dist_i           (AveragedLoss over the replica's B rows)
+ * and the total loss is the sum of the R replica losses (net.Sum, :236-238).  The gradient that
+ * enters the backward pass is d(total)/d(pred) = (pred - label) / B.  Rows [r*B, (r+1)*B) belong
+ * to replica r.  Accumulation in double; dY rounded to float once. */
+void oracle_l2_loss(int R, int B, int N, const float* pred, int ldp, const float* label, int ldl, float* dY, int lddy,
+                    double* loss_per_replica) {
+  const double inv_b = 1.0 / (double)B;
+  for (int r = 0; r < R; ++r) {
+    double acc = 0.0;
+    for (int i = r * B; i < (r + 1) * B; ++i) {
+      double dist = 0.0;
+      for (int j = 0; j < N; ++j) {
+        const double d = (double)pred[IDX(i, ldp, j)] - (double)label[IDX(i, ldl, j)];
+        dist += 0.5 * d * d;
+        if (dY) dY[IDX(i, lddy, j)] = (float)(d * inv_b);
+      }
+      acc += dist;
+    }
+    loss_per_replica[r] = acc * inv_b;
+  }
+}
+
 /* W[i] = fma(-lr, G_0[i] + G_1[i] + ... + G_{R-1}[i], W[i]) with fp32 adds in replica order and a
  * single-rounding fma, G_r = G + r*stride.  Arithmetic of mlp_omp.cc:140-143 (zmm add) and
  * :242-249 (add, then _mm512_fmadd_ps with -alpha rounded to float); R == 1 is :218-221. */

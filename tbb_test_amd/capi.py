@@ -80,6 +80,10 @@ SIGNATURES = {
     "mi_mlp_enable_timing": [c_void_p, c_int],
     "mi_mlp_reset_timings": [c_void_p],
     "mi_mlp_get_timings": [c_void_p, POINTER(c_double), POINTER(c_longlong)],
+    "mi_mlp_set_labels": [c_void_p, c_void_p, c_int],
+    "mi_loss_backward": [c_void_p],
+    "mi_mlp_get_loss": [c_void_p, POINTER(c_double), POINTER(c_double)],
+    "mi_mlp_trace_step": [c_void_p, c_float, c_char_p],
 }
 
 _lib = None
@@ -202,6 +206,25 @@ class MlpHandle:
         dY, p = _host_f32(dY)
         assert dY.shape == (self.MB, self.nf[self.L])
         check(lib().mi_mlp_set_dy(self._h, p, dY.shape[1]))
+
+    def set_labels(self, Y):
+        """Switches to loss mode: every step derives dY = (pred - Y) / B from its forward output."""
+        Y, p = _host_f32(Y)
+        assert Y.shape == (self.MB, self.nf[self.L])
+        check(lib().mi_mlp_set_labels(self._h, p, Y.shape[1]))
+
+    def loss(self):
+        """(loss_per_replica [R], total) of the last step in loss mode."""
+        per = (c_double * self.R)()
+        tot = c_double()
+        check(lib().mi_mlp_get_loss(self._h, per, ctypes.byref(tot)))
+        return np.array(per[:]), tot.value
+
+    def loss_backward(self): check(lib().mi_loss_backward(self._h))
+
+    def trace_step(self, lr, path):
+        """One step with an event pair around every launch; writes a Chrome-trace style timeline."""
+        check(lib().mi_mlp_trace_step(self._h, float(lr), os.fsencode(path)))
 
     # operations
     def forward(self, l): check(lib().mi_fc_forward(self._h, l))

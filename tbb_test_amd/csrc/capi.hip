@@ -85,6 +85,16 @@ struct mi_mlp {
 
   bool corun = false;  // set while enqueue_step issues the two backward chains on two streams
 
+  // loss front-end: when labels are set, every step derives dY from the forward output
+  float* labels = nullptr;         // [MB x nf[L]] fp32
+  double* loss_partials = nullptr; // [R x LOSS_CHUNKS] partial sums of 0.5 * (pred - label)^2 of the last step
+  bool use_loss = false;
+
+  // timeline of one step (mi_mlp_trace_step)
+  bool tracing = false;
+  struct TraceItem { hipEvent_t a, b; int breakdown, layer, stream_id; };
+  std::vector<TraceItem> trace_items;
+
   // timing
   bool timing = false;
   struct Pair { hipEvent_t a, b; int slot; };
@@ -145,23 +155,29 @@ int get_event(mi_mlp* h, hipEvent_t* ev) {
   return MI_OK;
 }
 
+constexpr int TRACE_LOSS = 100;   // pseudo-breakdown of the loss kernel in a timeline
+constexpr int LOSS_CHUNKS = 64;   // partial sums per replica
+
 struct TimedScope {
   mi_mlp* h;
   hipStream_t s;
   hipEvent_t a = nullptr, b = nullptr;
-  int slot;
+  int breakdown, layer;
   int status = MI_OK;
-  TimedScope(mi_mlp* h_, hipStream_t s_, int breakdown, int layer) : h(h_), s(s_), slot(breakdown * h_->L + layer) {
-    if (!h->timing) return;
+  bool on;
+  TimedScope(mi_mlp* h_, hipStream_t s_, int breakdown_, int layer_)
+      : h(h_), s(s_), breakdown(breakdown_), layer(layer_), on(h_->tracing || (h_->timing && breakdown_ < MI_NUM_BREAKDOWNS)) {
+    if (!on) return;
     if (h->pending.size() >= 8192) status = harvest(h);
     if (status == MI_OK) status = get_event(h, &a);
     if (status == MI_OK) status = get_event(h, &b);
     if (status == MI_OK && hipEventRecord(a, s) != hipSuccess) status = fail(MI_ERR_HIP, "hipEventRecord failed");
   }
   int finish() {
-    if (!h->timing || status != MI_OK) return status;
+    if (!on || status != MI_OK) return status;
     if (hipEventRecord(b, s) != hipSuccess) return fail(MI_ERR_HIP, "hipEventRecord failed");
-    h->pending.push_back({a, b, slot});
+    if (h->tracing) h->trace_items.push_back({a, b, breakdown, layer, s == h->stream ? 0 : 1});
+    else h->pending.push_back({a, b, breakdown * h->L + (layer < 0 ? 0 : layer)});
     return MI_OK;
   }
 };
@@ -261,7 +277,7 @@ int op_update(mi_mlp* h, int l_or_all, float lr, hipStream_t s) {
     n = (l_or_all + 1 < h->L ? h->woff[l_or_all + 1] : h->stride) - off;
     layer_slot = l_or_all;
   }
-  TimedScope ts(h, s, MI_WGT_UPDATE, layer_slot);
+  TimedScope ts(h, s, MI_WGT_UPDATE, l_or_all >= 0 ? layer_slot : -1);
   if (ts.status) return ts.status;
   hipError_t e = mi::reduce_sgd(h->params + off, h->params16 ? h->params16 + off : nullptr, h->grads + off, n,
                                 h->stride, h->R, lr, s);
@@ -297,6 +313,63 @@ int op_last_mask(mi_mlp* h, hipStream_t s) {
   return MI_OK;
 }
 
+// Loss front-end (SquaredL2Distance + AveragedLoss of the Caffe2 harness, mlp_caffe2.py:221-239):
+// dY = (pred - label) / B, and per replica the partial sums of 0.5 * (pred - label)^2.  Block
+// (c, r) owns a contiguous slice of replica r's elements; threads accumulate in double in a fixed
+// order and the block folds through LDS, so the result does not depend on scheduling.
+template <bool BF16>
+__global__ __launch_bounds__(256) void l2_loss_kernel(void* __restrict__ dy, const void* __restrict__ pred,
+                                                      const float* __restrict__ label, size_t per_replica,
+                                                      float inv_b, double* __restrict__ partials) {
+  __shared__ double red[256];
+  const size_t chunk = (per_replica + gridDim.x - 1) / gridDim.x;
+  const size_t lo = (size_t)blockIdx.y * per_replica + (size_t)blockIdx.x * chunk;
+  size_t hi = lo + chunk;
+  const size_t end = (size_t)(blockIdx.y + 1) * per_replica;
+  if (hi > end) hi = end;
+  double acc = 0.0;
+  for (size_t i = lo + threadIdx.x; i < hi; i += 256) {
+    float p;
+    if (BF16) p = __uint_as_float((unsigned)reinterpret_cast<const uint16_t*>(pred)[i] << 16);
+    else p = reinterpret_cast<const float*>(pred)[i];
+    const float d = p - label[i];
+    acc += 0.5 * (double)d * (double)d;
+    const float g = d * inv_b;
+    if (BF16) {
+      unsigned u = __float_as_uint(g);
+      if ((u & 0x7fffffffu) > 0x7f800000u) u = (u >> 16) | 0x40u;
+      else u = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+      reinterpret_cast<uint16_t*>(dy)[i] = (uint16_t)u;
+    } else {
+      reinterpret_cast<float*>(dy)[i] = g;
+    }
+  }
+  red[threadIdx.x] = acc;
+  __syncthreads();
+  for (int off = 128; off > 0; off >>= 1) {
+    if ((int)threadIdx.x < off) red[threadIdx.x] += red[threadIdx.x + off];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) partials[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = red[0];
+}
+
+int op_loss(mi_mlp* h, hipStream_t s) {
+  if (!h->labels) return fail(MI_ERR_INVALID, "no labels set (mi_mlp_set_labels)");
+  TimedScope ts(h, s, TRACE_LOSS, 0);
+  if (ts.status) return ts.status;
+  const size_t per_replica = (size_t)h->B * h->nf[h->L];
+  const float inv_b = 1.0f / (float)h->B;
+  if (h->dtype == MI_F32)
+    hipLaunchKernelGGL(l2_loss_kernel<false>, dim3(LOSS_CHUNKS, h->R), dim3(256), 0, s, h->dy, h->acts[h->L], h->labels,
+                       per_replica, inv_b, h->loss_partials);
+  else
+    hipLaunchKernelGGL(l2_loss_kernel<true>, dim3(LOSS_CHUNKS, h->R), dim3(256), 0, s, h->dy, h->acts[h->L], h->labels,
+                       per_replica, inv_b, h->loss_partials);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e, "loss launch");
+  return ts.finish();
+}
+
 // Enqueues one whole step.
 //
 // Backward runs on two streams: the input-gradient GEMMs form the dependent chain on the main
@@ -314,6 +387,8 @@ int enqueue_step(mi_mlp* h, float lr) {
   int rc;
   for (int l = 0; l < h->L; ++l)
     if ((rc = op_forward(h, l, s))) return rc;
+  if (h->use_loss)
+    if ((rc = op_loss(h, s))) return rc;
   if ((rc = op_last_mask(h, s))) return rc;
   // While per-kernel event timing is on, everything runs back to back on one stream with one
   // update launch: durations of kernels that overlap cannot be attributed to a kernel.
@@ -731,6 +806,12 @@ int mi_mlp_destroy(mi_mlp* h) {
   for (int i = 0; i < 3; ++i) (void)hipFree(h->dz[i]);
   (void)hipFree(h->dx);
   (void)hipFree(h->staging);
+  (void)hipFree(h->labels);
+  (void)hipFree(h->loss_partials);
+  for (auto& t : h->trace_items) {
+    (void)hipEventDestroy(t.a);
+    (void)hipEventDestroy(t.b);
+  }
   if (h->stream) (void)hipStreamDestroy(h->stream);
   if (h->stream2) (void)hipStreamDestroy(h->stream2);
   delete h;
@@ -765,7 +846,106 @@ int mi_mlp_set_input(mi_mlp* h, const float* X, int ld) {
 
 int mi_mlp_set_dy(mi_mlp* h, const float* dY, int ld) {
   if (int rc = check_handle(h)) return rc;
+  if (h->use_loss) {  // a given upstream gradient replaces the loss front-end
+    MI_HIP(hipStreamSynchronize(h->stream));
+    MI_HIP(hipStreamSynchronize(h->stream2));
+    h->use_loss = false;
+    drop_graph(h);
+  }
   return upload_matrix(h, h->dy, dY, h->MB, h->nf[h->L], ld, h->dtype == MI_BF16);
+}
+
+int mi_mlp_set_labels(mi_mlp* h, const float* Y, int ld) {
+  if (int rc = check_handle(h)) return rc;
+  MI_HIP(hipStreamSynchronize(h->stream));
+  MI_HIP(hipStreamSynchronize(h->stream2));
+  const size_t n = (size_t)h->MB * h->nf[h->L];
+  if (!h->labels) MI_HIP(hipMalloc((void**)&h->labels, n * 4));
+  if (!h->loss_partials) {
+    MI_HIP(hipMalloc((void**)&h->loss_partials, sizeof(double) * LOSS_CHUNKS * h->R));
+    MI_HIP(hipMemset(h->loss_partials, 0, sizeof(double) * LOSS_CHUNKS * h->R));
+  }
+  if (int rc = upload_matrix(h, h->labels, Y, h->MB, h->nf[h->L], ld, false)) return rc;
+  if (!h->use_loss) drop_graph(h);
+  h->use_loss = true;
+  return MI_OK;
+}
+
+int mi_loss_backward(mi_mlp* h) {
+  if (int rc = check_handle(h)) return rc;
+  return op_loss(h, h->stream);
+}
+
+int mi_mlp_get_loss(mi_mlp* h, double* loss_per_replica, double* total) {
+  if (int rc = check_handle(h)) return rc;
+  MI_REQUIRE(h->loss_partials != nullptr, "no labels set (mi_mlp_set_labels)");
+  MI_HIP(hipStreamSynchronize(h->stream));
+  MI_HIP(hipStreamSynchronize(h->stream2));
+  std::vector<double> part((size_t)LOSS_CHUNKS * h->R);
+  MI_HIP(hipMemcpy(part.data(), h->loss_partials, part.size() * sizeof(double), hipMemcpyDeviceToHost));
+  double sum = 0.0;
+  for (int r = 0; r < h->R; ++r) {
+    double acc = 0.0;
+    for (int c = 0; c < LOSS_CHUNKS; ++c) acc += part[(size_t)r * LOSS_CHUNKS + c];
+    acc /= (double)h->B;
+    if (loss_per_replica) loss_per_replica[r] = acc;
+    sum += acc;
+  }
+  if (total) *total = sum;
+  return MI_OK;
+}
+
+int mi_mlp_trace_step(mi_mlp* h, float lr, const char* path) {
+  if (int rc = check_handle(h)) return rc;
+  MI_REQUIRE(path != nullptr, "null path");
+  MI_REQUIRE(!h->timing, "per-kernel timing and the step timeline cannot be on together");
+  MI_HIP(hipStreamSynchronize(h->stream));
+  MI_HIP(hipStreamSynchronize(h->stream2));
+  hipEvent_t base = nullptr;
+  if (int rc = get_event(h, &base)) return rc;
+  h->tracing = true;
+  h->trace_items.clear();
+  int rc = MI_OK;
+  if (hipEventRecord(base, h->stream) != hipSuccess) rc = fail(MI_ERR_HIP, "hipEventRecord failed");
+  if (rc == MI_OK) rc = enqueue_step(h, lr);
+  h->tracing = false;
+  h->eager_steps++;
+  hipError_t e1 = hipStreamSynchronize(h->stream), e2 = hipStreamSynchronize(h->stream2);
+  if (rc == MI_OK && e1 != hipSuccess) rc = hip_fail(e1, "hipStreamSynchronize");
+  if (rc == MI_OK && e2 != hipSuccess) rc = hip_fail(e2, "hipStreamSynchronize");
+  FILE* f = rc == MI_OK ? fopen(path, "w") : nullptr;
+  if (rc == MI_OK && !f) rc = fail(MI_ERR_INVALID, "cannot open %s for writing", path);
+  if (f) {
+    // Same record layout as the reference's trace.log (mlp_tbb.cc:85-104,1379-1392): an array of
+    // begin/end records, ts in microseconds.  pid 0 is the GPU, tid the stream (0 main, 1 second).
+    static const char* kNames[] = {"FC", "FCWgtGradient", "FCBwdGradient", "ReduceScatterAllGather"};
+    fprintf(f, "[\n");
+    for (size_t i = 0; i < h->trace_items.size() && rc == MI_OK; ++i) {
+      const auto& t = h->trace_items[i];
+      float t0 = 0.0f, t1 = 0.0f;
+      if (hipEventElapsedTime(&t0, base, t.a) != hipSuccess || hipEventElapsedTime(&t1, base, t.b) != hipSuccess) {
+        rc = fail(MI_ERR_HIP, "hipEventElapsedTime failed");
+        break;
+      }
+      char name[64];
+      if (t.breakdown == TRACE_LOSS) snprintf(name, sizeof name, "L2Loss_0");
+      else if (t.layer < 0) snprintf(name, sizeof name, "%s_all_0", kNames[t.breakdown]);
+      else snprintf(name, sizeof name, "%s_%d_0", kNames[t.breakdown], t.layer);
+      fprintf(f, "{\n \"ts\": %.3f,\n \"pid\": 0,\n \"tid\": %d,\n \"name\": \"%s\",\n \"ph\": \"B\"\n},\n", t0 * 1e3,
+              t.stream_id, name);
+      fprintf(f, "{\n \"ts\": %.3f,\n \"pid\": 0,\n \"tid\": %d,\n \"ph\": \"E\"\n}%s\n", t1 * 1e3, t.stream_id,
+              i + 1 < h->trace_items.size() ? "," : "");
+    }
+    fprintf(f, "]\n");
+    fclose(f);
+  }
+  for (auto& t : h->trace_items) {
+    h->free_events.push_back(t.a);
+    h->free_events.push_back(t.b);
+  }
+  h->trace_items.clear();
+  h->free_events.push_back(base);
+  return rc;
 }
 
 int mi_fc_forward(mi_mlp* h, int l) {

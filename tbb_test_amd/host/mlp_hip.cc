@@ -14,6 +14,11 @@
 //   --no-graph    launch kernels one by one instead of replaying a captured HIP graph
 //   --keep-weights  let the weights evolve from step to step (default: every timed step starts
 //                 from the initial weights, so the values stay finite however many steps run)
+//   --loss l2     derive dY from seeded labels with SquaredL2Distance + AveragedLoss
+//                 (mlp_caffe2.py:221-239) instead of uploading a given dY; prints the loss
+//   --trace FILE  after the timed loop run one more step with an event pair around every launch
+//                 and write the timeline in the format of the reference's trace.log
+//                 (mlp_tbb.cc:1379-1392)
 #include <chrono>
 #include <cmath>
 #include <cstdio>
@@ -84,7 +89,7 @@ int main(int argc, char** argv) {
   if (argc < 2 || !isdigit((unsigned char)argv[1][0])) {
     fprintf(stderr, "%s <nreplicas> [nthreads_per_socket] [--config C1..C5|ref] [--layers L --width N --batch B] "
                     "[--lr X] [--seed S] [--warmup W] [--iters K] [--relu-last] [--overlap] [--no-graph] "
-                    "[--keep-weights]\n", argv[0]);
+                    "[--keep-weights] [--loss l2] [--trace FILE]\n", argv[0]);
     exit(1);
   }
   const int nreplicas_arg = atoi(argv[1]);
@@ -98,6 +103,7 @@ int main(int argc, char** argv) {
   uint64_t seed = 1;
   unsigned flags = 0;
   bool keep_weights = false, relu_last = false;
+  string loss, trace_path;
   for (; argi < argc; ++argi) {
     const string a = argv[argi];
     auto value = [&]() -> const char* {
@@ -116,6 +122,8 @@ int main(int argc, char** argv) {
     else if (a == "--overlap") flags |= MI_FLAG_PER_LAYER_UPDATE;
     else if (a == "--no-graph") flags |= MI_FLAG_NO_GRAPH;
     else if (a == "--keep-weights") keep_weights = true;
+    else if (a == "--loss") loss = value();
+    else if (a == "--trace") trace_path = value();
     else { fprintf(stderr, "unknown option %s\n", a.c_str()); exit(1); }
   }
 
@@ -163,7 +171,18 @@ int main(int argc, char** argv) {
   for (int l = 0; l < nlayers; ++l)
     MI_CHECK(mi_mlp_set_weights(h, l, weights[l]->rawData(), weights[l]->ld(), biases[l]->rawData()));
   MI_CHECK(mi_mlp_set_input(h, activations[0]->rawData(), activations[0]->ld()));
-  MI_CHECK(mi_mlp_set_dy(h, upstream_grad->rawData(), upstream_grad->ld()));
+  if (loss == "l2") {
+    // labels ~ U[-1, 1] on a stream of their own; the given dY is not used
+    Matrix<float, PAD> labels(R * B, model.nfeatures[nlayers]);
+    randStream(2000);
+    labels.randFill(-1.f, 1.f);
+    MI_CHECK(mi_mlp_set_labels(h, labels.rawData(), labels.ld()));
+  } else if (loss.empty()) {
+    MI_CHECK(mi_mlp_set_dy(h, upstream_grad->rawData(), upstream_grad->ld()));
+  } else {
+    fprintf(stderr, "unknown loss %s (known: l2)\n", loss.c_str());
+    exit(1);
+  }
   MI_CHECK(mi_mlp_snapshot_weights(h));
 
   size_t params = 0, stride = 0;
@@ -211,6 +230,21 @@ int main(int argc, char** argv) {
   printf("step %g ms, %g TFLOP/s over the whole step (GEMM FLOP model 3*2*batch*sum N_l*N_l+1 = %g GFLOP), "
          "update moves %g MB per step\n", step_ms, gemm_flop_step / step_ms / 1e9, gemm_flop_step / 1e9,
          (R + 2) * 4.0 * params / 1e6);
+
+  if (!loss.empty()) {
+    vector<double> per(R);
+    double total = 0;
+    MI_CHECK(mi_mlp_get_loss(h, per.data(), &total));
+    printf("loss %.9g (per replica:", total);
+    for (double v : per) printf(" %.9g", v);
+    printf(")\n");
+  }
+  if (!trace_path.empty()) {
+    MI_CHECK(mi_mlp_enable_timing(h, 0));
+    if (!keep_weights) MI_CHECK(mi_mlp_restore_weights(h));
+    MI_CHECK(mi_mlp_trace_step(h, model.lr, trace_path.c_str()));
+    printf("timeline of one step written to %s\n", trace_path.c_str());
+  }
 
   /////////////////////////////////////////////////////////////////////////////
   // print check sum for correctness check

@@ -4,6 +4,8 @@ What fixes each oracle function, besides its own formula:
   GEMMs            numpy float64 matmul (a library routine), identity / one-hot / sign special cases
   whole step       finite differences of the scalar <dY, output> in float64 (catches a dropped term,
                    a transposed operand, a wrong mask), R-replica split == one big batch
+  L2 loss          closed forms (zero at pred == label, constant offset), finite differences of the
+                   total loss in float64, independence of the replicas
   reduce + SGD     the reference's closed-form start-up check (mlp_omp.cc:325-373), R = 1 == plain
                    SGD, single-rounding of the fused multiply-add
   partition        fixture sweep produced by the compiled reference Partition.cc, the compiled
@@ -159,6 +161,51 @@ def test_step_replica_split_equals_one_big_batch():
 
 
 # ---- reduce + SGD ----------------------------------------------------------------------------------
+
+# ---- loss front-end ------------------------------------------------------------------------------
+
+def test_l2_loss_closed_forms():
+    R, B, N = 3, 4, 5
+    rng = np.random.default_rng(5)
+    label = rng.standard_normal((R * B, N)).astype(np.float32)
+    dY, loss = oracle.l2_loss(label, label, R)
+    assert np.all(dY == 0) and np.all(loss == 0)
+    # pred = label + c: every row is 0.5 c^2 N away, the mean over a replica is the same, dY = c / B
+    pred = (label.astype(np.float64) + 0.25).astype(np.float32)
+    exact = pred.astype(np.float64) - label
+    dY, loss = oracle.l2_loss(pred, label, R)
+    np.testing.assert_allclose(loss, [0.5 * (exact[r * B:(r + 1) * B] ** 2).sum() / B for r in range(R)], rtol=1e-14)
+    np.testing.assert_allclose(dY, exact / B, rtol=1e-6)
+    # a single wrong element in replica 1 changes only that replica's loss and that gradient entry
+    pred2 = label.copy()
+    pred2[B + 2, 3] += 2.0
+    dY, loss = oracle.l2_loss(pred2, label, R)
+    assert loss[0] == 0 and loss[2] == 0 and abs(loss[1] - 0.5 * 4.0 / B) < 1e-6
+    assert np.count_nonzero(dY) == 1 and abs(dY[B + 2, 3] - 2.0 / B) < 1e-6
+
+
+def test_l2_loss_gradient_matches_finite_differences():
+    R, B, N = 2, 3, 4
+    rng = np.random.default_rng(11)
+    pred = rng.standard_normal((R * B, N))
+    label = rng.standard_normal((R * B, N)).astype(np.float32)
+
+    def total(p):  # the definition, written independently in numpy float64
+        d = p - label.astype(np.float64)
+        return sum(0.5 * (d[r * B:(r + 1) * B] ** 2).sum() / B for r in range(R))
+
+    dY, loss = oracle.l2_loss(pred.astype(np.float32), label, R)
+    assert abs(loss.sum() - total(pred.astype(np.float32).astype(np.float64))) < 1e-12
+    eps = 1e-6
+    for (i, j) in [(0, 0), (2, 3), (3, 1), (5, 2)]:
+        hi, lo = pred.copy(), pred.copy()
+        hi[i, j] += eps
+        lo[i, j] -= eps
+        fd = (total(hi) - total(lo)) / (2 * eps)
+        assert abs(fd - dY[i, j]) < 1e-6, (i, j, fd, dY[i, j])
+
+
+# ---- reduce + SGD --------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("R", [1, 2, 3, 4, 8])
 def test_reduce_sgd_reference_known_answer(R):
