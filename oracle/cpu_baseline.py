@@ -1,5 +1,6 @@
-"""CPU baseline leg of bench.py: times the OpenMP restatement of the reference's mlp_omp
-(oracle/mlp_omp_port.c) on this host's cores.
+"""CPU baseline leg of bench.py: times the restatements of the reference's two CPU schedulers on
+this host's cores -- the OpenMP SPMD loop of mlp_omp (oracle/mlp_omp_port.c) and the task graph of
+mlp_tbb (oracle/mlp_dag_port.cc).
 
 TEST / MEASUREMENT INFRASTRUCTURE ONLY.  The number is a reported baseline, not a target.  The
 reference itself (MKL + TBB) cannot be built in this image, so the timed code is this repository's
@@ -30,6 +31,10 @@ def lib():
         l.port_mlp_run.argtypes = [_ci, ctypes.POINTER(_ci), _ci, _ci, _ci, ctypes.c_float, _ci, _vp, _vp, _vp, _ci,
                                    _ci, _ci, _vp, _vp, _vp, ctypes.POINTER(ctypes.c_double)]
         l.port_mlp_run.restype = _ci
+        l.port_mlp_dag_run.argtypes = l.port_mlp_run.argtypes
+        l.port_mlp_dag_run.restype = _ci
+        l.port_mlp_dag_comm_tasks.argtypes = [_ci]
+        l.port_mlp_dag_comm_tasks.restype = _ci
         l.port_check_all_reduce.argtypes = [_ci, _ci, _ci, _ci]
         l.port_check_all_reduce.restype = _ci
         l.port_partition_2d.argtypes = [_ci, _ci, ctypes.c_double, _ci, _ci, _ci, _ci, _ci, ctypes.POINTER(_ci)]
@@ -73,8 +78,10 @@ def host_cores():
     return max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
 
 
-def run_port(nf, B, R, T, lr, X, dY, W_flat, warmup, iters, restore=True, relu_last=False, use_blas=True):
-    """One call of the C port.  Returns (W_out flat, dX, times_ms[5])."""
+def run_port(nf, B, R, T, lr, X, dY, W_flat, warmup, iters, restore=True, relu_last=False, use_blas=True,
+             scheduler="omp"):
+    """One call of a port.  scheduler: "omp" (SPMD loop of mlp_omp) or "dag" (task graph of mlp_tbb).
+    Returns (W_out flat, dX, times_ms[5])."""
     L = len(nf) - 1
     MB = B * R
     X = np.ascontiguousarray(X, np.float32)
@@ -85,11 +92,12 @@ def run_port(nf, B, R, T, lr, X, dY, W_flat, warmup, iters, restore=True, relu_l
     times = (ctypes.c_double * 5)()
     arr = (_ci * len(nf))(*nf)
     sgemm = find_sgemm()[0] if use_blas else None
-    rc = lib().port_mlp_run(L, arr, B, R, T, lr, int(relu_last), X.ctypes.data_as(_vp), dY.ctypes.data_as(_vp),
-                            W_flat.ctypes.data_as(_vp), warmup, iters, int(restore), sgemm,
-                            W_out.ctypes.data_as(_vp), dX.ctypes.data_as(_vp), times)
+    fn = {"omp": lib().port_mlp_run, "dag": lib().port_mlp_dag_run}[scheduler]
+    rc = fn(L, arr, B, R, T, lr, int(relu_last), X.ctypes.data_as(_vp), dY.ctypes.data_as(_vp),
+            W_flat.ctypes.data_as(_vp), warmup, iters, int(restore), sgemm,
+            W_out.ctypes.data_as(_vp), dX.ctypes.data_as(_vp), times)
     if rc != 0:
-        raise RuntimeError(f"port_mlp_run failed with {rc}")
+        raise RuntimeError(f"{scheduler} port failed with {rc}")
     return W_out, dX, list(times)
 
 
@@ -105,10 +113,12 @@ def run(nf, B, R, lr, budget_s):
     W_flat = np.concatenate([np.concatenate([Ws[l].ravel(), bs[l].ravel()]) for l in range(L)])
     flop = 3 * 2.0 * R * B * sum(nf[l] * nf[l + 1] for l in range(L))
     _, _, t = run_port(nf, B, R, T, lr, X, dY, W_flat, 1, 1)          # warm caches, estimate the step time
-    iters = int(max(1, min(200, (budget_s - 2 * t[4] * 1e-3) / max(t[4] * 1e-3, 1e-6))))
+    # two thirds of the budget for the OpenMP restatement (the reported value), one third for the task graph
+    est = max(t[4] * 1e-3, 1e-6)
+    iters = int(max(1, min(200, (budget_s * 2 / 3 - 2 * est) / est)))
     _, _, t = run_port(nf, B, R, T, lr, X, dY, W_flat, 1, iters)
     ms = t[4]
-    return {
+    out = {
         "value": round(flop / (ms * 1e-3) / 1e12, 5),
         "unit": "TFLOP/s",
         "cores": R * T,
@@ -121,3 +131,13 @@ def run(nf, B, R, lr, budget_s):
                   f"{R} replicas x {T} threads = {R * T} OpenMP threads on {cores} host cores, restatement of "
                   "mlp_omp (oracle/mlp_omp_port.c)",
     }
+    dag_iters = int(max(1, min(100, (budget_s / 3 - est) / est)))
+    _, _, td = run_port(nf, B, R, T, lr, X, dY, W_flat, 1, dag_iters, scheduler="dag")
+    out["task_graph"] = {
+        "value": round(flop / (td[4] * 1e-3) / 1e12, 5),
+        "unit": "TFLOP/s",
+        "ms_per_step": round(td[4], 3),
+        "sample": f"{dag_iters} full step(s), {R} arenas x {T} threads, restatement of mlp_tbb's dependency graph "
+                  "(oracle/mlp_dag_port.cc)",
+    }
+    return out

@@ -113,8 +113,8 @@ void port_ring_info(int ns, int sid, int task, int out[3]) {
 /* ---- built-in SGEMM (used when no BLAS is supplied) ------------------------------------------ */
 /* C[m x n] = op(A) * op(B), row major, alpha = 1, beta = 0.  Plain k-blocked loops that the
  * compiler vectorises along n; adequate as a fallback, far from a tuned BLAS. */
-static void builtin_sgemm(int order, int ta, int tb, int m, int n, int k, float alpha, const float* a, int lda,
-                          const float* b, int ldb, float beta, float* c, int ldc) {
+void port_builtin_sgemm(int order, int ta, int tb, int m, int n, int k, float alpha, const float* a, int lda,
+                        const float* b, int ldb, float beta, float* c, int ldc) {
   (void)order; (void)alpha; (void)beta;
   enum { KB = 256 };
   float* bt = NULL;
@@ -294,7 +294,7 @@ static mat_t mat_alloc(int rows, int cols) {
 int port_mlp_run(int L, const int* nf, int B, int R, int T, float lr, int relu_last, const float* X, const float* dY,
                  const float* W_in, int warmup, int iters, int restore, cblas_sgemm_fn sgemm, float* W_out,
                  float* dX_out, double* times_ms) {
-  if (!sgemm) sgemm = builtin_sgemm;
+  if (!sgemm) sgemm = port_builtin_sgemm;
   const int MB = R * B, nthreads = R * T;
   mat_t* act = (mat_t*)calloc((size_t)L + 2, sizeof(mat_t));
   mat_t *wt = (mat_t*)calloc((size_t)L, sizeof(mat_t)), *gr = (mat_t*)calloc((size_t)L, sizeof(mat_t)),
