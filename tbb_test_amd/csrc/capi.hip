@@ -83,7 +83,7 @@ struct mi_mlp {
   std::vector<hipEvent_t> ev_layer;  // per layer: input-gradient GEMM of layer l done (dZ_{l-1} ready, W_l free)
   std::vector<hipEvent_t> ev_wgrad;  // per layer: weight-gradient GEMM of layer l done (dZ_l free)
 
-  bool corun = false;  // set while enqueue_step issues the two backward chains on two streams
+  bool corun = false;  // set while enqueue_step issues an input-gradient GEMM next to a short-K weight gradient
 
   // loss front-end: when labels are set, every step derives dY from the forward output
   float* labels = nullptr;         // [MB x nf[L]] fp32
@@ -215,7 +215,7 @@ int op_wgrad(mi_mlp* h, int l, hipStream_t s, bool with_bias) {
     e = mi::sgemm_tn(h->R, h->nf[l + 1], h->nf[l], h->B, (const float*)dz_of_layer(h, l), h->nf[l + 1],
                      (const float*)h->acts[l], h->nf[l], const_cast<float*>(g0), h->nf[l], (long long)h->stride,
                      with_bias ? h->grads + h->boff[l] : nullptr, (long long)h->stride, s,
-                     g_variant[2] ? g_variant[2] : (h->corun ? 100 : 0));
+                     g_variant[2]);
   } else {
     // K-contiguous copies of both operands, per replica: A_l^T [N_l x B] and dZ_l^T [N_{l+1} x B]
     const int B = h->B, nin = h->nf[l], nout = h->nf[l + 1];
@@ -399,10 +399,11 @@ int enqueue_step(mi_mlp* h, float lr) {
     MI_HIP(hipEventRecord(h->ev_fork, s));
     MI_HIP(hipStreamWaitEvent(s2, h->ev_fork, 0));
   }
-  // The backward GEMMs of a layer are told when they run next to each other with about one tile
-  // per CU each (then the kernels with the small LDS footprint share CUs).  The hint follows the
-  // configured schedule, not the momentary one, so that the per-kernel timing pass measures the
-  // kernels the real step uses.
+  // The input-gradient GEMM of a layer is told when a weight-gradient GEMM with a short K (small
+  // per-replica batch) runs next to it on the second stream; it then takes the kernel with the
+  // larger LDS footprint so that it keeps its share of every CU.  The hint follows the configured
+  // schedule, not the momentary one, so that the per-kernel timing pass measures the kernels the
+  // real step uses.
   struct CorunScope {
     mi_mlp* h;
     explicit CorunScope(mi_mlp* h_) : h(h_) {}
@@ -410,8 +411,7 @@ int enqueue_step(mi_mlp* h, float lr) {
   } corun_scope(h);
   const bool corun_cfg = !(h->flags & MI_FLAG_SERIAL_BACKWARD);
   for (int l = h->L - 1; l >= 0; --l) {
-    const long long wgrad_tiles = (long long)(h->nf[l + 1] / 128) * (h->nf[l] / 128) * h->R;
-    h->corun = corun_cfg && wgrad_tiles < 512;
+    h->corun = corun_cfg && h->B < 512;
     if ((rc = op_wgrad(h, l, s2, true))) return rc;
     if (dual) {
       MI_HIP(hipEventRecord(h->ev_wgrad[l], s2));

@@ -539,27 +539,12 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     else variant = -1;
   }
   switch (variant) {
-    case 1: if (fits(256, 256, 32)) return launch_h<256, 256, 32, 2, 2, EPI>(p, batch, s); break;
-    case 2: if (fits(256, 128, 32)) return launch_h<256, 128, 32, 2, 2, EPI>(p, batch, s); break;
     case 3: if (fits(128, 128, 32)) return launch_h<128, 128, 32, 2, 2, EPI>(p, batch, s); break;
     case 4: if (fits(256, 256, 32)) return launch_h<256, 256, 32, 2, 4, EPI>(p, batch, s); break;
     case 5: if (fits(64, 64, 32)) return launch_h<64, 64, 32, 2, 2, EPI>(p, batch, s); break;
-    case 6: if (fits(128, 128, 64)) return launch_h<128, 128, 64, 2, 2, EPI>(p, batch, s); break;
-    case 7: if (fits(256, 256, 64)) return launch_h<256, 256, 64, 2, 2, EPI, 1, 2>(p, batch, s); break;
-    case 8: if (fits(256, 256, 32)) return launch_h<256, 256, 32, 2, 4, EPI, 2>(p, batch, s); break;
-    case 9: if (fits(256, 256, 64)) return launch_h<256, 256, 64, 2, 4, EPI, 1, 2>(p, batch, s); break;
-    case 10: if (fits(256, 128, 64)) return launch_h<256, 128, 64, 2, 2, EPI, 1, 3>(p, batch, s); break;
-    case 11: if (fits(256, 128, 64)) return launch_h<256, 128, 64, 2, 4, EPI, 1, 3>(p, batch, s); break;
-    case 12: if (fits(128, 256, 64)) return launch_h<128, 256, 64, 2, 4, EPI, 1, 3>(p, batch, s); break;
     case 13: if (fits(256, 256, 32)) return launch_dma<256, 256, 32, 2, 4, EPI, 4>(p, batch, s); break;
-    case 14: if (fits(256, 256, 32)) return launch_dma<256, 256, 32, 2, 4, EPI, 3>(p, batch, s); break;
-    case 15: if (fits(256, 256, 32)) return launch_dma<256, 256, 32, 2, 2, EPI, 4>(p, batch, s); break;
-    case 16: if (fits(256, 128, 64)) return launch_dma<256, 128, 64, 2, 4, EPI, 3>(p, batch, s); break;
     case 17: if (fits(128, 128, 32)) return launch_dma<128, 128, 32, 2, 2, EPI, 4>(p, batch, s); break;
-    case 18: if (fits(128, 128, 64)) return launch_dma<128, 128, 64, 2, 2, EPI, 4>(p, batch, s); break;
     case 19: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2>(p, batch, s); break;
-    case 20: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 4, 2, EPI, 2>(p, batch, s); break;
-    case 21: if (fits(256, 256, 32)) return launch_dma<256, 256, 32, 2, 4, EPI, 5>(p, batch, s); break;
     default: break;
   }
   hipLaunchKernelGGL((gemm_bf16_generic<EPI>), dim3((p.N + 15) / 16, (p.M + 15) / 16, batch), dim3(256), 0, s, p);

@@ -220,6 +220,88 @@ __device__ __forceinline__ void load_frag(float (&frag)[TB][4], const float* lds
   }
 }
 
+// ---- epilogue: registers -> global, fused bias/ReLU or ReLU mask ------------------------------
+// Writes the TM x TN accumulator blocks of one wavefront; (m0w, n0w) is the wavefront's first
+// row / column in C.
+template <int TM, int TN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool GUARD>
+__device__ __forceinline__ void write_tile(const GemmArgs& p, float* __restrict__ C, f32x16 (&acc)[TM][TN], int m0w,
+                                           int n0w, int lane) {
+  // Column of (block j, value e) held by this lane: K-major B keeps the blocks side by side,
+  // N-major B interleaves them so that the lane owns TN consecutive columns (one vector store).
+  const int l32 = lane & 31, hi = lane >> 5;
+  const int col0 = n0w + (B_KMAJOR ? l32 : TN * l32);
+  constexpr int CSTEP = B_KMAJOR ? 32 : 1;
+  const float* __restrict__ mask = p.mask;
+
+  // GUARD: element (row, column j of this lane) exists
+  auto col_ok = [&](int j) { return !GUARD || col0 + j * CSTEP < p.N; };
+  constexpr bool VEC_STORE = !B_KMAJOR && (TN == 2 || TN == 4);
+  // a vector access covers TN consecutive columns starting at col0; with GUARD it needs all of them
+  const bool vec_ok = VEC_STORE && (!GUARD || ((p.vec_flags & 4) && col0 + TN - 1 < p.N));
+
+  float bias_v[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+    bias_v[j] = (EPI == EPI_BIAS_RELU && p.bias && col_ok(j)) ? p.bias[col0 + j * CSTEP] : 0.0f;
+
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    // rows of accumulator registers r = 0..15 of block row i
+    auto row_of = [&](int r) {
+      const int rb32 = 8 * (r >> 2) + 4 * hi + (r & 3);
+      return m0w + (A_KMAJOR ? i * 32 + rb32 : TM * rb32 + i);
+    };
+    // all mask reads of this block row first, so that they are in flight together
+    float mk[16][TN];
+    if (EPI == EPI_MASK) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = row_of(r);
+        const float* mrow = mask + (size_t)row * p.ldmask + col0;
+        const bool row_ok = !GUARD || row < p.M;
+        if (VEC_STORE && TN == 4 && vec_ok && row_ok) {
+          const f32x4 t = *reinterpret_cast<const f32x4*>(mrow);
+          mk[r][0] = t[0]; mk[r][1 % TN] = t[1]; mk[r][2 % TN] = t[2]; mk[r][3 % TN] = t[3];
+        } else if (VEC_STORE && TN == 2 && vec_ok && row_ok) {
+          const f32x2 t = *reinterpret_cast<const f32x2*>(mrow);
+          mk[r][0] = t[0]; mk[r][1 % TN] = t[1];
+        } else {
+#pragma unroll
+          for (int j = 0; j < TN; ++j) mk[r][j] = (row_ok && col_ok(j)) ? mrow[j * CSTEP] : 0.0f;
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = row_of(r);
+      if (GUARD && row >= p.M) continue;
+      float* crow = C + (size_t)row * p.ldc + col0;
+      float v[TN];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        v[j] = acc[i][j][r];
+        if (EPI == EPI_BIAS_RELU) {
+          v[j] += bias_v[j];
+          if (p.relu) v[j] = v[j] > 0.0f ? v[j] : 0.0f;
+        } else if (EPI == EPI_MASK) {
+          if (!(mk[r][j] > 0.0f)) v[j] = 0.0f;
+        }
+      }
+      if (VEC_STORE && TN == 4 && vec_ok) {
+        const f32x4 o = {v[0], v[1 % TN], v[2 % TN], v[3 % TN]};
+        *reinterpret_cast<f32x4*>(crow) = o;
+      } else if (VEC_STORE && TN == 2 && vec_ok) {
+        const f32x2 o = {v[0], v[1 % TN]};
+        *reinterpret_cast<f32x2*>(crow) = o;
+      } else {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          if (col_ok(j)) crow[j * CSTEP] = v[j];
+      }
+    }
+  }
+}
+
 // COLSUM (weight gradient only, A stored [k][m]): the workgroups of tile column 0 also add up the
 // columns of their A tile while it sits in LDS.  Every thread takes part so that no wavefront
 // falls behind: thread t owns column t % BM and the k rows of slice t / BM of every K step; the
@@ -446,81 +528,221 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
     }
   }
 
-  // ---- epilogue: registers -> global, fused bias/ReLU or ReLU mask --------------------------
-  // Column of (block j, value e) held by this lane: K-major B keeps the blocks side by side,
-  // N-major B interleaves them so that the lane owns TN consecutive columns (one vector store).
+  write_tile<TM, TN, A_KMAJOR, B_KMAJOR, EPI, GUARD>(p, C, acc, m0 + wm0, n0 + wn0, lane);
+}
+
+// ---- the same GEMM with direct global -> LDS loads ----------------------------------------------
+// global_load_lds_dwordx4 moves 16 bytes per lane from global memory straight into the LDS: the 64
+// lanes of one instruction fill 1 KB of consecutive LDS bytes from a wave-uniform base (lane i
+// lands at base + 16 i) while every lane names its own global address.  The tile no longer passes
+// through VGPRs: the ds_write of the next tile and the wait for its global loads at the top of
+// every K step -- measured at 7 % of the register-staged kernel's time -- disappear.
+//
+// LDS layouts (no padding, an instruction's 1 KB must be contiguous):
+//   K-major operand  [row][BK]; the 16-byte chunk c of row r sits at chunk position c ^ swz(r),
+//                    swz(r) = (r / rows per 256 bytes) mod chunks per row.  The swizzle is produced
+//                    on the global side (the lane that fills position pc of row r fetches chunk
+//                    pc ^ swz(r)); the 16 lanes the LDS serves together on a fragment read (same
+//                    chunk, 16 consecutive rows) then touch all 64 banks once.
+//   M-major operand  [k][ROWS], as in the register-staged kernel.
+//
+// Ring of STAGES buffers; in the middle of step t every wave waits (vmcnt) until its own loads of
+// tile t+1 have landed, all waves meet at one barrier, and the loads of tile t+STAGES-1 are issued
+// into the buffer step t-1 read.  The load is inline assembly on purpose: the compiler models the
+// builtin as a FLAT access that may touch both memories and then turns every later LDS-counter
+// wait into lgkmcnt(0) while such a load is pending; written this way it does not track the load
+// at all and the kernel counts vmcnt itself (compiler-inserted vmcnt waits can only get longer
+// through the extra loads in flight, never shorter: vmcnt retires in order).
+__device__ __forceinline__ void load_to_lds_f32(const float* src, unsigned lds_byte_addr) {
+  const unsigned lds_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr);
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory", "m0");
+}
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
+// expcnt 6:4, lgkmcnt 11:8; the other counters at their maximum = no wait).
+constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | 0x70 | 0xf00; }
+
+template <int ROWS, int BK>
+struct SwizzledTile {
+  static constexpr int kChunks = BK / 4;                                   // 16-byte chunks per row
+  static constexpr int kRowsPerLine = 256 / (BK * 4) > 0 ? 256 / (BK * 4) : 1;
+  static __device__ __forceinline__ int swz(int row) { return (row / kRowsPerLine) % kChunks; }
+};
+
+// K-major fragment read from the swizzled layout: same values as load_frag<.., true, ..>.
+template <int ROWS, int BK, int TB>
+__device__ __forceinline__ void load_frag_swz(float (&frag)[TB][4], const float* lds, int wave_row0, int kk, int lane) {
+  using ST = SwizzledTile<ROWS, BK>;
   const int l32 = lane & 31, hi = lane >> 5;
-  const int col0 = n0 + wn0 + (B_KMAJOR ? l32 : TN * l32);
-  constexpr int CSTEP = B_KMAJOR ? 32 : 1;
-  const float* __restrict__ mask = p.mask;
+#pragma unroll
+  for (int b = 0; b < TB; ++b) {
+    const int row = wave_row0 + b * 32 + l32;
+    const f32x4 t = *reinterpret_cast<const f32x4*>(lds + row * BK + ((kk * 2 + hi) ^ ST::swz(row)) * 4);
+    frag[b][0] = t[0];
+    frag[b][1] = t[1];
+    frag[b][2] = t[2];
+    frag[b][3] = t[3];
+  }
+}
 
-  // GUARD: element (row, column j of this lane) exists
-  auto col_ok = [&](int j) { return !GUARD || col0 + j * CSTEP < p.N; };
-  constexpr bool VEC_STORE = !B_KMAJOR && (TN == 2 || TN == 4);
-  // a vector access covers TN consecutive columns starting at col0; with GUARD it needs all of them
-  const bool vec_ok = VEC_STORE && (!GUARD || ((p.vec_flags & 4) && col0 + TN - 1 < p.N));
+template <int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM, int STAGES,
+          bool PIN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
+  constexpr int NW = WM * WN, NT = NW * 64;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int CH = BK / 8;
+  constexpr int A_FLOATS = BM * BK, B_FLOATS = BN * BK;
+  // load instructions per wave and tile: an instruction covers 1 KB = 256 floats of the tile
+  constexpr int NIA = A_FLOATS / 256 / NW, NIB = B_FLOATS / 256 / NW, INSTR = NIA + NIB;
+  static_assert(STAGES >= 3 && STAGES <= 5, "ring depth");
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0 && CH % 2 == 0, "tile shape");
+  static_assert(A_FLOATS % (256 * NW) == 0 && B_FLOATS % (256 * NW) == 0, "tile must divide over the waves");
+  static_assert((STAGES - 2) * INSTR <= 63, "vmcnt is a 6-bit counter");
+  static_assert(A_KMAJOR || TM == 1 || TM == 2 || TM == 4, "interleaved A needs TM in {1,2,4}");
+  static_assert(B_KMAJOR || TN == 1 || TN == 2 || TN == 4, "interleaved B needs TN in {1,2,4}");
+  static_assert(!COLSUM || (!A_KMAJOR && NT % BM == 0 && BK % (NT / BM) == 0),
+                "fused column sums need A stored [k][m] and a whole number of k slices");
 
-  float bias_v[TN];
-#pragma unroll
-  for (int j = 0; j < TN; ++j)
-    bias_v[j] = (EPI == EPI_BIAS_RELU && p.bias && col_ok(j)) ? p.bias[col0 + j * CSTEP] : 0.0f;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  auto As = [&](int buf) { return smem + buf * A_FLOATS; };
+  auto Bs = [&](int buf) { return smem + STAGES * A_FLOATS + buf * B_FLOATS; };
+  const unsigned lds_base = (unsigned)(size_t)((__attribute__((address_space(3))) const void*)smem);
 
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    // rows of accumulator registers r = 0..15 of block row i
-    auto row_of = [&](int r) {
-      const int rb32 = 8 * (r >> 2) + 4 * hi + (r & 3);
-      return m0 + wm0 + (A_KMAJOR ? i * 32 + rb32 : TM * rb32 + i);
-    };
-    // all mask reads of this block row first, so that they are in flight together
-    float mk[16][TN];
-    if (EPI == EPI_MASK) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = row_of(r);
-        const float* mrow = mask + (size_t)row * p.ldmask + col0;
-        const bool row_ok = !GUARD || row < p.M;
-        if (VEC_STORE && TN == 4 && vec_ok && row_ok) {
-          const f32x4 t = *reinterpret_cast<const f32x4*>(mrow);
-          mk[r][0] = t[0]; mk[r][1 % TN] = t[1]; mk[r][2 % TN] = t[2]; mk[r][3 % TN] = t[3];
-        } else if (VEC_STORE && TN == 2 && vec_ok && row_ok) {
-          const f32x2 t = *reinterpret_cast<const f32x2*>(mrow);
-          mk[r][0] = t[0]; mk[r][1 % TN] = t[1];
-        } else {
-#pragma unroll
-          for (int j = 0; j < TN; ++j) mk[r][j] = (row_ok && col_ok(j)) ? mrow[j * CSTEP] : 0.0f;
-        }
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
+
+  int tile_m, tile_n;
+  tile_of_block(p, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  float* __restrict__ C = p.C + (size_t)blockIdx.z * p.batchC;
+
+  // global source of this lane for each of its load instructions, and the advance per K step
+  const float* ga[NIA];
+  const float* gb[NIB];
+  auto sources = [&](auto& g, auto kmajor, auto rows_c, const float* op, int ld, int first_row, int ni) {
+    constexpr bool KM = decltype(kmajor)::value;
+    constexpr int ROWS = decltype(rows_c)::value;
+    for (int j = 0; j < ni; ++j) {
+      const int unit = j * NW + wave;  // which 1 KB piece of the tile
+      if (KM) {
+        using ST = SwizzledTile<ROWS, BK>;
+        constexpr int RPI = 64 / ST::kChunks;
+        const int row = unit * RPI + lane / ST::kChunks, pc = lane % ST::kChunks;
+        g[j] = op + (size_t)(first_row + row) * ld + (pc ^ ST::swz(row)) * 4;
+      } else {
+        constexpr int CPR = ROWS / 4, KPI = 64 / CPR > 0 ? 64 / CPR : 1;
+        static_assert(CPR <= 64, "a tile row must fit one load instruction");
+        const int k = unit * KPI + lane / CPR, c = lane % CPR;
+        g[j] = op + (size_t)k * ld + first_row + c * 4;
       }
     }
+  };
+  sources(ga, std::integral_constant<bool, A_KMAJOR>{}, std::integral_constant<int, BM>{},
+          p.A + (size_t)blockIdx.z * p.batchA, p.lda, m0, NIA);
+  sources(gb, std::integral_constant<bool, B_KMAJOR>{}, std::integral_constant<int, BN>{},
+          p.B + (size_t)blockIdx.z * p.batchB, p.ldb, n0, NIB);
+  const size_t a_step = A_KMAJOR ? (size_t)BK : (size_t)BK * p.lda;
+  const size_t b_step = B_KMAJOR ? (size_t)BK : (size_t)BK * p.ldb;
+  auto issue = [&](int buf) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = row_of(r);
-      if (GUARD && row >= p.M) continue;
-      float* crow = C + (size_t)row * p.ldc + col0;
-      float v[TN];
+    for (int j = 0; j < NIA; ++j) {
+      load_to_lds_f32(ga[j], lds_base + 4u * (unsigned)(buf * A_FLOATS + (j * NW + wave) * 256));
+      ga[j] += a_step;
+    }
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        v[j] = acc[i][j][r];
-        if (EPI == EPI_BIAS_RELU) {
-          v[j] += bias_v[j];
-          if (p.relu) v[j] = v[j] > 0.0f ? v[j] : 0.0f;
-        } else if (EPI == EPI_MASK) {
-          if (!(mk[r][j] > 0.0f)) v[j] = 0.0f;
-        }
+    for (int j = 0; j < NIB; ++j) {
+      load_to_lds_f32(gb[j], lds_base + 4u * (unsigned)(STAGES * A_FLOATS + buf * B_FLOATS + (j * NW + wave) * 256));
+      gb[j] += b_step;
+    }
+  };
+  auto frags = [&](float (&fa)[TM][4], float (&fb)[TN][4], int buf, int kk) {
+    if constexpr (A_KMAJOR) load_frag_swz<BM, BK, TM>(fa, As(buf), wm0, kk, lane);
+    else load_frag<BM, BK, false, TM>(fa, As(buf), wm0, kk, lane);
+    if constexpr (B_KMAJOR) load_frag_swz<BN, BK, TN>(fb, Bs(buf), wn0, kk, lane);
+    else load_frag<BN, BK, false, TN>(fb, Bs(buf), wn0, kk, lane);
+  };
+  // Barrier of the ring.  Nothing is written with ds_write, so no LDS-counter wait is needed for
+  // visibility; a buffer is refilled only after the MFMAs that consumed its last fragments.  The
+  // fused column sums read the tile with plain LDS loads whose consumers the compiler may delay,
+  // so that instantiation drains the LDS counter first.
+  auto ring_barrier = [&]() {
+    if constexpr (COLSUM) __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0) only
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  constexpr int CS_SLICES = COLSUM ? NT / BM : 1;
+  constexpr int CS_ROWS = BK / CS_SLICES;
+  const bool do_colsum = COLSUM && p.colsum != nullptr && tile_n == 0;
+  float csum = 0.0f;
+
+  const int nk = p.K / BK;
+#pragma unroll
+  for (int st = 0; st < STAGES - 1; ++st)
+    if (st < nk) issue(st);
+  if (nk >= STAGES - 1) __builtin_amdgcn_s_waitcnt(vmcnt_only((STAGES - 2) * INSTR));
+  else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+  ring_barrier();
+
+  float fa[2][TM][4], fb[2][TN][4];
+  frags(fa[0], fb[0], 0, 0);
+  int cur = 0;
+  for (int t = 0; t < nk; ++t) {
+    const int nxt = cur + 1 == STAGES ? 0 : cur + 1;
+    const int fill = cur == 0 ? STAGES - 1 : cur - 1;
+#pragma unroll
+    for (int kk = 0; kk < CH; ++kk) {
+      const int fc = kk & 1, fn = fc ^ 1;
+      if (kk + 1 < CH) frags(fa[fn], fb[fn], cur, kk + 1);
+      else frags(fa[fn], fb[fn], nxt, 0);  // after the last tile: a harmless read of ring memory, keeps one code path
+      if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[fc][i][q], fb[fc][j][q], acc[i][j], 0, 0, 0);
+      if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+      if (kk == CH - 2) {
+        // tiles t+1 .. t+STAGES-2 are in flight; tile t+1 must have landed
+        if (t + STAGES - 2 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_only((STAGES - 3) * INSTR));
+        else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+        ring_barrier();
+        if (t + STAGES - 1 < nk) issue(fill);
       }
-      if (VEC_STORE && TN == 4 && vec_ok) {
-        const f32x4 o = {v[0], v[1 % TN], v[2 % TN], v[3 % TN]};
-        *reinterpret_cast<f32x4*>(crow) = o;
-      } else if (VEC_STORE && TN == 2 && vec_ok) {
-        const f32x2 o = {v[0], v[1 % TN]};
-        *reinterpret_cast<f32x2*>(crow) = o;
-      } else {
+      if (kk == CH - 1 && COLSUM && do_colsum) {
+        const float* col = As(cur) + (tid / BM) * CS_ROWS * BM + (tid % BM);
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          if (col_ok(j)) crow[j * CSTEP] = v[j];
+        for (int k = 0; k < CS_ROWS; ++k) csum += col[k * BM];
       }
+    }
+    cur = nxt;
+  }
+
+  if (COLSUM && do_colsum) {
+    __syncthreads();  // every wavefront is done with the operand tiles: reuse LDS for the partials
+    smem[tid] = csum;
+    __syncthreads();
+    if (tid < BM) {
+      float total = smem[tid];
+#pragma unroll
+      for (int sl = 1; sl < CS_SLICES; ++sl) total += smem[sl * BM + tid];
+      p.colsum[(size_t)blockIdx.z * p.batchColsum + m0 + tid] = total;
     }
   }
+  write_tile<TM, TN, A_KMAJOR, B_KMAJOR, EPI, false>(p, C, acc, m0 + wm0, n0 + wn0, lane);
 }
 
 // ---- any-shape fallback ----------------------------------------------------------------------
@@ -610,6 +832,24 @@ static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
   return hipGetLastError();
 }
 
+template <int BM, int BN, int BK, int WM, int WN, bool AK, bool BKM, int EPI, bool COLSUM, int STAGES, bool PIN = false>
+static hipError_t launch_dma(GemmArgs& p, int batch, hipStream_t s) {
+  constexpr size_t lds_bytes = STAGES * (size_t)(BM + BN) * BK * sizeof(float);
+  static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB of LDS");
+  auto kern = gemm_f32_dma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES, PIN>;
+  static bool attr_set = false;
+  if (lds_bytes > 64 * 1024 && !attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  p.tiles_m = p.M / BM;
+  p.tiles_n = p.N / BN;
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
+  return hipGetLastError();
+}
+
 template <bool AK, bool BKM, int EPI>
 static hipError_t launch_generic(GemmArgs& p, int batch, hipStream_t s) {
   dim3 grid((p.N + 63) / 64, (p.M + 63) / 64, batch);
@@ -633,23 +873,28 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
   auto fits = [&](int bm, int bn, int bk) {
     return vec_ok && mask_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0;
   };
-  // variant 100 = automatic, and the caller runs another GEMM next to this one on a second stream:
-  // then the 61 KB kernel pays off from one tile per CU on, because workgroups of the two kernels
-  // share CUs.
+  // variant 100 = automatic, and the caller runs a weight-gradient GEMM with a short K next to
+  // this one on a second stream (see below).
   const bool corun = variant == 100;
   if (corun) variant = 0;
   if (variant == 0) {
-    // Automatic choice among the 8-wavefront, 3-stage kernels on 128 x 128 tiles.  With two or more
-    // tiles per CU take BK = 16: its three LDS buffers are 61 KB, so two workgroups share a CU and
-    // one's prologue, epilogue and barrier waits are covered by the other's MFMAs.  With about one
-    // tile per CU nothing can overlap, and BK = 32 (110 KB, one workgroup per CU, half as many
-    // barriers) is faster.  Smaller problems fall back to 128 x 64 and 64 x 64 tiles to get
-    // enough workgroups.
+    // Automatic choice.  From about one 128 x 128 tile per CU on, the direct-to-LDS kernels with a
+    // ring of three buffers: BK = 16 (48 KB, up to three workgroups share a CU and one's prologue,
+    // epilogue and barrier waits are covered by another's MFMAs) or BK = 32 (96 KB, one workgroup
+    // per CU, half as many barriers).  Measured on the benchmark configurations, whole step:
+    //   * forward and input gradient: BK = 16;
+    //   * weight gradient (with its fused column sums): BK = 32 from K = 512 on, BK = 16 for the
+    //     short K of small per-replica batches;
+    //   * an input-gradient GEMM that runs next to such a short-K weight gradient takes BK = 32:
+    //     with 48 KB each, two weight-gradient workgroups would sit beside every input-gradient
+    //     workgroup and slow the chain of dependent input-gradient GEMMs that bounds the step.
+    // Smaller problems fall back to 128 x 64 and 64 x 64 tiles to get enough workgroups.
     const long long tiles128 = (long long)(p.M / 128) * (p.N / 128) * batch;
-    if (fits(128, 128, 32) && (tiles128 >= 512 || (corun && tiles128 >= 192))) {
-      variant = 10;
-    } else if (fits(128, 128, 32) && tiles128 >= 192) {
-      variant = 8;
+    constexpr bool kWeightGradient = !AK && !BKM;
+    if (fits(128, 128, 32) && tiles128 >= 192 && ((kWeightGradient && p.K >= 512) || corun)) {
+      variant = 31;
+    } else if (fits(128, 128, 16) && tiles128 >= 192) {
+      variant = 33;
     } else if (fits(128, 64, 32) && tiles128 * 2 >= 192) {
       variant = 11;
     } else if (fits(64, 64, 16)) {
@@ -667,28 +912,22 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
                 ((aligned16(p.B) && p.ldb % 4 == 0 && p.batchB % 4 == 0) ? 2 : 0) |
                 ((aligned16(p.C) && p.ldc % 4 == 0 && p.batchC % 4 == 0 && mask_ok) ? 4 : 0);
   switch (variant) {
-    case 1: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
-    case 2: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
-    case 3: if (fits(256, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<256, 128, 32, 2, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
-    case 4: if (fits(64, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<64, 64, 32, 2, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
-    case 5: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 16, 2, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
-    case 6: if (fits(256, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<256, 128, 16, 4, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
-    case 7: if (fits(128, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI, COLSUM>(p, batch, s); } break;
     case 8: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 9: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 10: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 11: if (fits(128, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 12: if (fits(128, 64, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 16, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
-    case 13: if (fits(64, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<64, 128, 16, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
-    case 14: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 16, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 15: if (fits(128, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI, COLSUM, 2>(p, batch, s); } break;
     case 16: if (fits(64, 64, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<64, 64, 16, 2, 2, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 17: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 3, 2>(p, batch, s); } break;
-    case 18: if (fits(128, 64, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 64, 32, 2, 2, AK, BKM, EPI, COLSUM, 3, 2>(p, batch, s); } break;
-    case 19: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3, 2>(p, batch, s); } break;
-    case 20: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 2, AK, BKM, EPI, COLSUM, 3, 2>(p, batch, s); } break;
     case 21: if (p.K > 0) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 3, 1, true>(p, batch, s); } break;
     case 22: if (p.K > 0) { if (fused_colsum) *fused_colsum = COLSUM; return launch_mfma<64, 64, 16, 2, 2, AK, BKM, EPI, COLSUM, 3, 1, true>(p, batch, s); } break;
+    case 30: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 4>(p, batch, s); } break;
+    case 31: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 32: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 4>(p, batch, s); } break;
+    case 33: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 34: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 4, true>(p, batch, s); } break;
+    case 35: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 4, true>(p, batch, s); } break;
     default: break;
   }
   return launch_generic<AK, BKM, EPI>(p, batch, s);

@@ -53,7 +53,7 @@ def test_bf16_helpers_round_to_nearest_even():
 
 HSHAPES = [(64, 64, 32), (128, 128, 64), (256, 256, 96), (512, 256, 128), (256, 512, 32), (7, 5, 9), (100, 130, 50),
            (129, 64, 40), (256, 256, 512)]
-HVARIANTS = list(range(0, 22))
+HVARIANTS = [0, 3, 4, 5, 13, 17, 19]
 
 
 @pytest.mark.parametrize("variant", HVARIANTS)
