@@ -16,9 +16,11 @@ Prints one JSON line:
                  3 * 2 * (R*B) * sum_l N_l*N_{l+1}   (mlp_omp.cc:492,584,675)
   ms_per_step    wall clock of the timed loop / K
   roofline       the GEMM kernels (the dominant kernels): FLOP per launch / average launch
-                 duration from HIP events on the launching stream, against the fp32 MFMA peak.
-                 Taken in a second pass over the same K steps in which every kernel runs alone
-                 (one stream, one update launch): overlapping kernels cannot be timed individually
+                 duration, against the fp32 MFMA peak.  Durations come from HIP events attached
+                 to each kernel dispatch on the stream it is launched on (start and stop event of
+                 hipExtLaunchKernelGGL), in a second pass over the same K steps in which every
+                 kernel runs alone (one stream, one update launch): overlapping kernels cannot be
+                 timed individually
   roofline_reduce  the reduce+SGD kernel: (R+2)*4*P bytes / its launch duration, against HBM peak
   cpu_baseline   the CPU restatement of the reference's mlp_omp timed on this host's cores
 """
@@ -45,8 +47,7 @@ METRIC = "MLP fwd+bwd+reduce step ms & TFLOP/s on 1 MI355X; grad-reduce GB/s"
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark
 # (FETCH_SIZE scaled by 1.9986, WRITE_SIZE by 1.0, the factors a plain 33.6 MB device copy gives;
-# the runs are summarised under profiles/; the BK = 16 kernels the default schedule uses for the
-# backward GEMMs read the same panels as the BK = 32 kernels these were taken on).  GEMM: mean over the forward, weight-gradient and
+# the runs are summarised under profiles/).  GEMM: mean over the forward, weight-gradient and
 # input-gradient launches.  None = not measured for that configuration.
 MEASURED_TRAFFIC_BYTES = {
     "C2": {"gemm": (50.4e6 + 16.8e6 + 151.0e6 + 16.8e6 + 67.2e6 + 16.8e6) / 3, "reduce": 167.8e6 + 33.6e6},
@@ -174,7 +175,7 @@ def main():
         "gemm_tflops": round(gemm_tflops, 2),
         "reduce_gbps": round(upd_gbps, 1),
         "weights_finite": finite,
-        "roofline": {"kernel": "gemm_f32_mfma (nt, nn, tn)" if dtype == "f32" else "gemm_bf16_mfma",
+        "roofline": {"kernel": "gemm_f32_dma (nt, nn, tn)" if dtype == "f32" else "gemm_bf16_dma",
                      "bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(gemm_tflops / peak, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get("gemm"),

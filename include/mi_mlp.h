@@ -238,7 +238,8 @@ int mi_mlp_param_count(mi_mlp* h, size_t* params, size_t* replica_stride);
 /*
  * Per-phase device timing with HIP events on the handle's stream (the role of sum_times /
  * dsecnd() in mlp_omp.cc:490-508,582-600,673-691,161-168).  While enabled, every kernel of
- * mi_mlp_step and of the per-operation entry points is bracketed by an event pair.
+ * mi_mlp_step and of the per-operation entry points carries a start and a stop event on its
+ * dispatch, so the figures are kernel execution times without launch gaps.
  * While timing is enabled the step runs serially on one stream with a single update launch,
  * whatever the scheduling flags say, because overlapping kernels cannot be timed individually.
  * mi_mlp_get_timings synchronises and writes accumulated milliseconds as

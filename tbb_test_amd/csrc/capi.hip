@@ -161,7 +161,7 @@ constexpr int LOSS_CHUNKS = 64;   // partial sums per replica
 struct TimedScope {
   mi_mlp* h;
   hipStream_t s;
-  hipEvent_t a = nullptr, b = nullptr;
+  mi::LaunchEvents ev{nullptr, nullptr, 0};
   int breakdown, layer;
   int status = MI_OK;
   bool on;
@@ -169,15 +169,23 @@ struct TimedScope {
       : h(h_), s(s_), breakdown(breakdown_), layer(layer_), on(h_->tracing || (h_->timing && breakdown_ < MI_NUM_BREAKDOWNS)) {
     if (!on) return;
     if (h->pending.size() >= 8192) status = harvest(h);
-    if (status == MI_OK) status = get_event(h, &a);
-    if (status == MI_OK) status = get_event(h, &b);
-    if (status == MI_OK && hipEventRecord(a, s) != hipSuccess) status = fail(MI_ERR_HIP, "hipEventRecord failed");
+    if (status == MI_OK) status = get_event(h, &ev.start);
+    if (status == MI_OK) status = get_event(h, &ev.stop);
+    if (status == MI_OK) mi::launch_events = &ev;  // the kernels of this scope carry the events
+  }
+  ~TimedScope() {
+    if (mi::launch_events == &ev) mi::launch_events = nullptr;
   }
   int finish() {
     if (!on || status != MI_OK) return status;
-    if (hipEventRecord(b, s) != hipSuccess) return fail(MI_ERR_HIP, "hipEventRecord failed");
-    if (h->tracing) h->trace_items.push_back({a, b, breakdown, layer, s == h->stream ? 0 : 1});
-    else h->pending.push_back({a, b, breakdown * h->L + (layer < 0 ? 0 : layer)});
+    mi::launch_events = nullptr;
+    if (ev.launches == 0) {  // nothing was launched (empty operand): nothing to time
+      h->free_events.push_back(ev.start);
+      h->free_events.push_back(ev.stop);
+      return MI_OK;
+    }
+    if (h->tracing) h->trace_items.push_back({ev.start, ev.stop, breakdown, layer, s == h->stream ? 0 : 1});
+    else h->pending.push_back({ev.start, ev.stop, breakdown * h->L + (layer < 0 ? 0 : layer)});
     return MI_OK;
   }
 };
@@ -306,7 +314,7 @@ int op_last_mask(mi_mlp* h, hipStream_t s) {
   const size_t n = (size_t)h->MB * h->nf[h->L];
   size_t blocks = (n + 255) / 256;
   if (blocks > 4096) blocks = 4096;
-  hipLaunchKernelGGL(mask_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float*)h->dz[(h->L - 1) % 3],
+  mi::launch_kernel(mask_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float*)h->dz[(h->L - 1) % 3],
                      (const float*)h->dy, (const float*)h->acts[h->L], n);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e, "mask launch");
@@ -360,10 +368,10 @@ int op_loss(mi_mlp* h, hipStream_t s) {
   const size_t per_replica = (size_t)h->B * h->nf[h->L];
   const float inv_b = 1.0f / (float)h->B;
   if (h->dtype == MI_F32)
-    hipLaunchKernelGGL(l2_loss_kernel<false>, dim3(LOSS_CHUNKS, h->R), dim3(256), 0, s, h->dy, h->acts[h->L], h->labels,
+    mi::launch_kernel(l2_loss_kernel<false>, dim3(LOSS_CHUNKS, h->R), dim3(256), 0, s, h->dy, h->acts[h->L], h->labels,
                        per_replica, inv_b, h->loss_partials);
   else
-    hipLaunchKernelGGL(l2_loss_kernel<true>, dim3(LOSS_CHUNKS, h->R), dim3(256), 0, s, h->dy, h->acts[h->L], h->labels,
+    mi::launch_kernel(l2_loss_kernel<true>, dim3(LOSS_CHUNKS, h->R), dim3(256), 0, s, h->dy, h->acts[h->L], h->labels,
                        per_replica, inv_b, h->loss_partials);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e, "loss launch");

@@ -499,7 +499,7 @@ static hipError_t launch_h(HGemmArgs& p, int batch, hipStream_t s) {
   }
   p.tiles_m = p.M / BM;
   p.tiles_n = p.N / BN;
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
+  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
   return hipGetLastError();
 }
 
@@ -517,7 +517,7 @@ static hipError_t launch_dma(HGemmArgs& p, int batch, hipStream_t s) {
   }
   p.tiles_m = p.M / BM;
   p.tiles_n = p.N / BN;
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
+  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
   return hipGetLastError();
 }
 
@@ -547,7 +547,7 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     case 19: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2>(p, batch, s); break;
     default: break;
   }
-  hipLaunchKernelGGL((gemm_bf16_generic<EPI>), dim3((p.N + 15) / 16, (p.M + 15) / 16, batch), dim3(256), 0, s, p);
+  launch_kernel((gemm_bf16_generic<EPI>), dim3((p.N + 15) / 16, (p.M + 15) / 16, batch), dim3(256), 0, s, p);
   return hipGetLastError();
 }
 
@@ -591,7 +591,7 @@ __global__ __launch_bounds__(256) void transpose16_kernel(u16* __restrict__ dst,
 hipError_t transpose_bf16(int batch, int rows, int cols, const uint16_t* src, int ld_src, long long batch_src,
                           uint16_t* dst, int ld_dst, long long batch_dst, hipStream_t s) {
   if (batch <= 0 || rows <= 0 || cols <= 0) return hipSuccess;
-  hipLaunchKernelGGL(transpose16_kernel, dim3((cols + 63) / 64, (rows + 63) / 64, batch), dim3(256), 0, s, dst, src, rows,
+  launch_kernel(transpose16_kernel, dim3((cols + 63) / 64, (rows + 63) / 64, batch), dim3(256), 0, s, dst, src, rows,
                      cols, ld_src, ld_dst, batch_src, batch_dst);
   return hipGetLastError();
 }
@@ -613,7 +613,7 @@ __global__ __launch_bounds__(256) void rowsum16_kernel(float* __restrict__ out, 
 hipError_t rowsum_bf16(int batch, int rows, int cols, const uint16_t* src, int ld, long long batch_src, float* out,
                        long long stride_out, hipStream_t s) {
   if (batch <= 0 || rows <= 0) return hipSuccess;
-  hipLaunchKernelGGL(rowsum16_kernel, dim3((rows + 3) / 4, batch), dim3(256), 0, s, out, src, rows, cols, ld, batch_src,
+  launch_kernel(rowsum16_kernel, dim3((rows + 3) / 4, batch), dim3(256), 0, s, out, src, rows, cols, ld, batch_src,
                      stride_out);
   return hipGetLastError();
 }

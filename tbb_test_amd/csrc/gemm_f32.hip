@@ -828,7 +828,7 @@ static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
   p.tiles_m = GUARD ? (p.M + BM - 1) / BM : p.M / BM;
   p.tiles_n = GUARD ? (p.N + BN - 1) / BN : p.N / BN;
   dim3 grid(p.tiles_m * p.tiles_n, 1, batch);
-  hipLaunchKernelGGL(kern, grid, dim3(WM * WN * 64), lds_bytes, s, p);
+  launch_kernel(kern, grid, dim3(WM * WN * 64), lds_bytes, s, p);
   return hipGetLastError();
 }
 
@@ -846,14 +846,14 @@ static hipError_t launch_dma(GemmArgs& p, int batch, hipStream_t s) {
   }
   p.tiles_m = p.M / BM;
   p.tiles_n = p.N / BN;
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
+  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
   return hipGetLastError();
 }
 
 template <bool AK, bool BKM, int EPI>
 static hipError_t launch_generic(GemmArgs& p, int batch, hipStream_t s) {
   dim3 grid((p.N + 63) / 64, (p.M + 63) / 64, batch);
-  hipLaunchKernelGGL((gemm_f32_generic<AK, BKM, EPI>), grid, dim3(256), 0, s, p);
+  launch_kernel((gemm_f32_generic<AK, BKM, EPI>), grid, dim3(256), 0, s, p);
   return hipGetLastError();
 }
 

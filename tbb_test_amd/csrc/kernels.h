@@ -3,11 +3,38 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstddef>
 #include <cstdint>
 
 namespace mi {
+
+// Per-launch timing.  While `launch_events` is set (by the timing scope of the C ABI, on the
+// calling thread), kernels are launched through hipExtLaunchKernelGGL with a start and a stop
+// event attached to the dispatch itself: the pair then measures the kernel's own execution, as a
+// profiler's kernel trace does, and not the gap to the previous kernel that a hipEventRecord
+// before the launch would add.  The first launch of a scope takes the start event, every launch
+// re-records the stop event, so a scope of several kernels is timed from the first kernel's
+// start to the last kernel's end.
+struct LaunchEvents {
+  hipEvent_t start, stop;
+  int launches;
+};
+extern thread_local LaunchEvents* launch_events;
+
+template <typename... KArgs, typename... Args>
+inline void launch_kernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t s,
+                          Args... args) {
+  LaunchEvents* ev = launch_events;
+  if (ev) {
+    hipEvent_t start = ev->launches == 0 ? ev->start : nullptr;
+    ev->launches++;
+    hipExtLaunchKernelGGL(kernel, grid, block, (std::uint32_t)lds_bytes, s, start, ev->stop, 0, static_cast<KArgs>(args)...);
+  } else {
+    hipLaunchKernelGGL(kernel, grid, block, lds_bytes, s, static_cast<KArgs>(args)...);
+  }
+}
 
 // `variant` selects a tile configuration of the MFMA kernel (0 = choose from the shape, 100 =
 // choose from the shape knowing that another GEMM runs concurrently on a second stream); it is

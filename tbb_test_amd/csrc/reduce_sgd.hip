@@ -13,6 +13,8 @@
 
 namespace mi {
 
+thread_local LaunchEvents* launch_events = nullptr;
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
 
@@ -118,10 +120,10 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
 #define MI_LAUNCH_REDUCE2(RF, BF)                                                                          \
   do {                                                                                                     \
     if (stream)                                                                                            \
-      hipLaunchKernelGGL((reduce_sgd_vec4<RF, BF, 1, true>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, \
+      launch_kernel((reduce_sgd_vec4<RF, BF, 1, true>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, \
                          stride / 4, R, neg_lr);                                                           \
     else                                                                                                   \
-      hipLaunchKernelGGL((reduce_sgd_vec4<RF, BF, 2, false>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, \
+      launch_kernel((reduce_sgd_vec4<RF, BF, 2, false>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, \
                          stride / 4, R, neg_lr);                                                           \
   } while (0)
 #define MI_LAUNCH_REDUCE(RF, BF) MI_LAUNCH_REDUCE2(RF, BF)
@@ -150,7 +152,7 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
   }
   if (done < n) {
     const int blocks = grid_for(n - done, 256, 2048);
-    hipLaunchKernelGGL(reduce_sgd_scalar, dim3(blocks), dim3(256), 0, s, W, W16, G, done, n, stride, R, neg_lr);
+    launch_kernel(reduce_sgd_scalar, dim3(blocks), dim3(256), 0, s, W, W16, G, done, n, stride, R, neg_lr);
   }
   return hipGetLastError();
 }
@@ -179,7 +181,7 @@ __global__ __launch_bounds__(256) void colsum_kernel(int M, int K, const float* 
 hipError_t colsum_f32(int R, int M, int K, const float* A, int lda, float* out, long long stride_out,
                       hipStream_t s) {
   if (R <= 0 || M <= 0) return hipSuccess;
-  hipLaunchKernelGGL(colsum_kernel, dim3((M + 63) / 64, R), dim3(256), 0, s, M, K, A, lda, out, stride_out);
+  launch_kernel(colsum_kernel, dim3((M + 63) / 64, R), dim3(256), 0, s, M, K, A, lda, out, stride_out);
   return hipGetLastError();
 }
 
@@ -199,13 +201,13 @@ __global__ __launch_bounds__(256) void bf16_to_f32_kernel(float* __restrict__ ds
 
 hipError_t convert_f32_to_bf16(uint16_t* dst, const float* src, size_t n, hipStream_t s) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(grid_for(n, 256, 4096)), dim3(256), 0, s, dst, src, n);
+  launch_kernel(f32_to_bf16_kernel, dim3(grid_for(n, 256, 4096)), dim3(256), 0, s, dst, src, n);
   return hipGetLastError();
 }
 
 hipError_t convert_bf16_to_f32(float* dst, const uint16_t* src, size_t n, hipStream_t s) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(bf16_to_f32_kernel, dim3(grid_for(n, 256, 4096)), dim3(256), 0, s, dst, src, n);
+  launch_kernel(bf16_to_f32_kernel, dim3(grid_for(n, 256, 4096)), dim3(256), 0, s, dst, src, n);
   return hipGetLastError();
 }
 
