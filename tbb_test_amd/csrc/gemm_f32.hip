@@ -1,4 +1,4 @@
-// fp32 GEMM kernels for gfx950 on v_mfma_f32_32x32x2_f32, one template for the three operand
+// fp32 GEMM kernels for gfx950 on v_mfma_f32_32x32x2_f32, templates over the three operand
 // layouts of the MLP step:
 //   NT  C = A[M,K] * B[N,K]^T   forward        (reference call site mlp_omp.cc:474-488)
 //   NN  C = A[M,K] * B[K,N]     input gradient (mlp_omp.cc:657-671)
@@ -6,16 +6,17 @@
 //
 // Structure of one workgroup (WM x WN wavefronts of 64 lanes):
 //   - owns a BM x BN tile of C; walks K in steps of BK;
-//   - global -> registers -> LDS with two LDS buffers, so the loads of step t+1 are in flight
-//     while step t is multiplied (one barrier per step);
+//   - operand tiles travel global -> LDS either directly (gemm_f32_dma: global_load_lds into a
+//     ring of LDS buffers; the kernel of all large GEMMs) or through registers (gemm_f32_mfma:
+//     small tilings, and the guarded instances for ragged or unaligned shapes);
 //   - each wavefront owns a (BM/WM) x (BN/WN) sub-tile as TM x TN blocks of 32 x 32 held in
 //     accumulator registers.
 //
 // Operand fragments.  One MFMA consumes, per lane, one A value A[i = lane%32][k = lane/32] and
 // one B value B[k = lane/32][j = lane%32].  A lane fetches four values with one 16-byte LDS
 // read, and what the four values are depends on how the operand lies in memory:
-//   * "K-major" operand (k contiguous: A of NT/NN, B of NT): the tile is stored [row][k] with
-//     a 4-float pad per row; the lane reads k = kk*8 + 4*(lane/32) + {0,1,2,3} of its row and
+//   * "K-major" operand (k contiguous: A of NT/NN, B of NT): the tile is stored [row][k] (with
+//     a 4-float pad per row in gemm_f32_mfma, XOR-swizzled chunks in gemm_f32_dma); the lane reads k = kk*8 + 4*(lane/32) + {0,1,2,3} of its row and
 //     feeds them to four consecutive MFMAs of the same 32 x 32 block.
 //   * "M-major" operand (rows contiguous: A of TN, B of NN/TN): the tile is stored [k][row];
 //     the lane reads rows TM*(lane%32) + {0..TM-1} of one k and feeds them to the TM blocks of
