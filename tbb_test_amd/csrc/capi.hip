@@ -71,7 +71,11 @@ struct mi_mlp {
   uint16_t* params16_saved = nullptr;
   uint16_t* params16T_saved = nullptr;
   std::vector<uint16_t*> actsT;  // bf16 only: per-replica transposed activations [R][N_l x B], l < L
-  uint16_t* dzT = nullptr;       // bf16 only: per-replica transposed gradient [R][max N x B]
+  // bf16 only: per-replica transposed gradients [R][max N x B]; dZ_l^T lives in dzT[l % 3] like
+  // dZ_l in dz[l % 3].  *_fused: the producing GEMM wrote the transposed copy in its epilogue.
+  uint16_t* dzT[3] = {nullptr, nullptr, nullptr};
+  std::vector<char> actsT_fused;  // [L]
+  bool dzT_fused[3] = {false, false, false};
   std::vector<void*> acts;    // L+1 buffers [MB x nf[l]], fp32 or bf16
   void* dy = nullptr;         // upstream gradient [MB x nf[L]]
   void* dz[3] = {nullptr, nullptr, nullptr};  // gradient rotation [MB x max width]: dZ_l lives in dz[l % 3]
@@ -206,9 +210,13 @@ int op_forward(mi_mlp* h, int l, hipStream_t s) {
     e = mi::sgemm_nt(h->MB, h->nf[l + 1], h->nf[l], (const float*)h->acts[l], h->nf[l], h->params + h->woff[l],
                      h->nf[l], (float*)h->acts[l + 1], h->nf[l + 1], h->params + h->boff[l], relu, s, g_variant[0]);
   } else {
+    // the activation a later weight-gradient GEMM reads K-contiguous is also written transposed
+    bool wrote = false;
+    uint16_t* ct = (l + 1 < h->L) ? h->actsT[l + 1] : nullptr;
     e = mi::hgemm_nt(1, h->MB, h->nf[l + 1], h->nf[l], (const uint16_t*)h->acts[l], h->nf[l], 0,
                      h->params16 + h->woff[l], h->nf[l], 0, h->acts[l + 1], h->nf[l + 1], 0, 1, h->params + h->boff[l],
-                     relu, nullptr, 0, s, g_hvariant);
+                     relu, nullptr, 0, s, g_hvariant, ct, h->B, &wrote);
+    if (l + 1 < h->L) h->actsT_fused[l + 1] = wrote;
   }
   if (e != hipSuccess) return hip_fail(e, "forward GEMM launch");
   return ts.finish();
@@ -227,16 +235,22 @@ int op_wgrad(mi_mlp* h, int l, hipStream_t s, bool with_bias) {
   } else {
     // K-contiguous copies of both operands, per replica: A_l^T [N_l x B] and dZ_l^T [N_{l+1} x B]
     const int B = h->B, nin = h->nf[l], nout = h->nf[l + 1];
-    e = mi::transpose_bf16(h->R, B, nin, (const uint16_t*)h->acts[l], nin, (long long)B * nin, h->actsT[l], B,
-                           (long long)nin * B, s);
-    if (e == hipSuccess)
-      e = mi::transpose_bf16(h->R, B, nout, (const uint16_t*)dz_of_layer(h, l), nout, (long long)B * nout, h->dzT, B,
+    // (each copy comes from the epilogue of the GEMM that produced the operand when that was
+    // possible, else from a transpose here)
+    uint16_t* dzt = h->dzT[l % 3];
+    e = hipSuccess;
+    if (!h->actsT_fused[l])
+      e = mi::transpose_bf16(h->R, B, nin, (const uint16_t*)h->acts[l], nin, (long long)B * nin, h->actsT[l], B,
+                             (long long)nin * B, s);
+    const bool dz_fused = l < h->L - 1 && h->dzT_fused[l % 3];  // the last layer's dZ is the given or derived dY
+    if (e == hipSuccess && !dz_fused)
+      e = mi::transpose_bf16(h->R, B, nout, (const uint16_t*)dz_of_layer(h, l), nout, (long long)B * nout, dzt, B,
                              (long long)nout * B, s);
     if (e == hipSuccess)
-      e = mi::hgemm_nt(h->R, nout, nin, B, h->dzT, B, (long long)nout * B, h->actsT[l], B, (long long)nin * B,
+      e = mi::hgemm_nt(h->R, nout, nin, B, dzt, B, (long long)nout * B, h->actsT[l], B, (long long)nin * B,
                        const_cast<float*>(g0), nin, (long long)h->stride, 0, nullptr, 0, nullptr, 0, s, g_hvariant);
     if (e == hipSuccess && with_bias)
-      e = mi::rowsum_bf16(h->R, nout, B, h->dzT, B, (long long)nout * B, h->grads + h->boff[l], (long long)h->stride, s);
+      e = mi::rowsum_bf16(h->R, nout, B, dzt, B, (long long)nout * B, h->grads + h->boff[l], (long long)h->stride, s);
   }
   if (e != hipSuccess) return hip_fail(e, "weight-gradient GEMM launch");
   return ts.finish();
@@ -246,9 +260,10 @@ int op_bgrad(mi_mlp* h, int l, hipStream_t s) {
   if (h->dtype != MI_F32) {
     const int B = h->B, nout = h->nf[l + 1];
     hipError_t eb = mi::transpose_bf16(h->R, B, nout, (const uint16_t*)dz_of_layer(h, l), nout, (long long)B * nout,
-                                       h->dzT, B, (long long)nout * B, s);
+                                       h->dzT[l % 3], B, (long long)nout * B, s);
     if (eb == hipSuccess)
-      eb = mi::rowsum_bf16(h->R, nout, B, h->dzT, B, (long long)nout * B, h->grads + h->boff[l], (long long)h->stride, s);
+      eb = mi::rowsum_bf16(h->R, nout, B, h->dzT[l % 3], B, (long long)nout * B, h->grads + h->boff[l],
+                           (long long)h->stride, s);
     if (eb != hipSuccess) return hip_fail(eb, "bias-gradient launch");
     return MI_OK;
   }
@@ -269,9 +284,12 @@ int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
                      h->params + h->woff[l], h->nf[l], (float*)out, h->nf[l], (const float*)mask, h->nf[l], s,
                      g_variant[1] ? g_variant[1] : (h->corun ? 100 : 0));
   } else {
+    bool wrote = false;
+    uint16_t* ct = (l > 0) ? h->dzT[(l - 1) % 3] : nullptr;  // dZ_{l-1}^T for the weight gradient of layer l-1
     e = mi::hgemm_nt(1, h->MB, h->nf[l], h->nf[l + 1], (const uint16_t*)dz_of_layer(h, l), h->nf[l + 1], 0,
                      h->params16T + h->woff[l], h->nf[l + 1], 0, out, h->nf[l], 0, mask ? 2 : 3, nullptr, 0,
-                     (const uint16_t*)mask, h->nf[l], s, g_hvariant);
+                     (const uint16_t*)mask, h->nf[l], s, g_hvariant, ct, h->B, &wrote);
+    if (l > 0) h->dzT_fused[(l - 1) % 3] = wrote;
   }
   if (e != hipSuccess) return hip_fail(e, "input-gradient GEMM launch");
   return ts.finish();
@@ -748,7 +766,8 @@ int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_repli
     alloc((void**)&h->params16T, h->stride * 2);
     h->actsT.assign(L, nullptr);
     for (int l = 0; l < L; ++l) alloc((void**)&h->actsT[l], (size_t)h->MB * h->nf[l] * 2);
-    alloc((void**)&h->dzT, (size_t)h->MB * h->maxw() * 2);
+    for (int i = 0; i < 3; ++i) alloc((void**)&h->dzT[i], (size_t)h->MB * h->maxw() * 2);
+    h->actsT_fused.assign(L, 0);
     size_t wmax = 0;
     for (int l = 0; l < L; ++l) wmax = std::max(wmax, (size_t)h->nf[l] * h->nf[l + 1]);
     h->staging_elems = std::max((size_t)h->MB * h->maxw(), wmax);
@@ -808,7 +827,7 @@ int mi_mlp_destroy(mi_mlp* h) {
   (void)hipFree(h->params16T);
   (void)hipFree(h->params16T_saved);
   for (auto a : h->actsT) (void)hipFree(a);
-  (void)hipFree(h->dzT);
+  for (int i = 0; i < 3; ++i) (void)hipFree(h->dzT[i]);
   for (void* a : h->acts) (void)hipFree(a);
   (void)hipFree(h->dy);
   for (int i = 0; i < 3; ++i) (void)hipFree(h->dz[i]);

@@ -46,6 +46,11 @@ struct HGemmArgs {
   const u16* mask;  // bf16 [M x N]: result zeroed where mask <= 0
   int ldmask;
   int tiles_m, tiles_n;
+  // optional second output (bf16 epilogues): the same values transposed per group of ct_rows
+  // rows, Ct[(row / ct_rows)][col][row % ct_rows] with row stride ct_rows and N * ct_rows elements
+  // per group -- the K-contiguous per-replica copy the weight-gradient GEMM reads
+  u16* Ct;
+  int ct_rows;
 };
 
 __device__ __forceinline__ u16 f2bf(float f) {
@@ -89,15 +94,26 @@ __device__ __forceinline__ void tile_of_workgroup(int id, int tiles_m, int tiles
 
 // Writes a wavefront's TM x TN accumulator blocks (32 x 32 each) with the epilogue EPI.  Lane l,
 // register r of a block hold row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+//
+// Transposed second output (p.Ct).  Registers 4g .. 4g+3 of a block are four consecutive rows of
+// one column, i.e. 8 contiguous bytes of the transposed copy.  Stored straight from the registers
+// these are 8-byte pieces scattered over 32 columns per instruction, which the write path handles
+// badly (measured: +160 us on a 1.8 ms GEMM).  With `lds` != nullptr (the caller guarantees the
+// workgroup's LDS is free and gives each wavefront its own region of 32 * (TM*64 + 8) bytes) the
+// pieces go through the LDS instead, one 32-column block at a time, columns padded by 8 bytes so
+// that the 32 lanes of a half-wave hit distinct banks, and are read back as 16-byte chunks: one
+// store instruction then writes whole runs of TM*64 contiguous bytes.
 template <int TM, int TN, int EPI>
 __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[TM][TN], int row0, int colw, int l32,
-                                             int hi) {
+                                             int hi, u16* lds = nullptr) {
+  typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
   const int col0 = colw + l32;
   float bias_v[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j) bias_v[j] = (EPI == EPH_BIAS_RELU && p.bias) ? p.bias[col0 + j * 32] : 0.0f;
   float* __restrict__ cf = reinterpret_cast<float*>(p.C) + (size_t)blockIdx.z * p.batchC;
   u16* __restrict__ ch = reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC;
+  unsigned pk[TM][TN][8];  // bf16 results, two rows per register: (4g, 4g+1) and (4g+2, 4g+3)
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -116,9 +132,53 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
           } else if (EPI == EPH_MASK) {
             if (!(bf2f(p.mask[(size_t)row * p.ldmask + col]) > 0.0f)) v = 0.0f;
           }
-          ch[(size_t)row * p.ldc + col] = f2bf(v);
+          const u16 o = f2bf(v);
+          ch[(size_t)row * p.ldc + col] = o;
+          if (r & 1) pk[i][j][r >> 1] |= (unsigned)o << 16;
+          else pk[i][j][r >> 1] = o;
         }
       }
+    }
+  }
+  if (EPI == EPH_F32 || !p.Ct) return;
+  // the tile lies inside one row group: ct_rows is a multiple of the tile height
+  const int group = row0 / p.ct_rows, m_local0 = row0 - group * p.ct_rows;
+  u16* __restrict__ ct = p.Ct + (size_t)group * p.N * p.ct_rows + m_local0;
+  if (lds == nullptr) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        u16* dst = ct + (size_t)(col0 + j * 32) * p.ct_rows + i * 32 + 4 * hi;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const u32x2 two = {pk[i][j][2 * g], pk[i][j][2 * g + 1]};
+          *reinterpret_cast<u32x2*>(dst + 8 * g) = two;
+        }
+      }
+    return;
+  }
+  constexpr int COL_BYTES = TM * 64 + 8;  // TM*32 rows of bf16 plus the pad
+  constexpr int CHUNKS = TM * 4;          // 16-byte chunks per column
+  const int lane = hi * 32 + l32;
+  unsigned char* region = reinterpret_cast<unsigned char*>(lds);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const u32x2 two = {pk[i][j][2 * g], pk[i][j][2 * g + 1]};
+        *reinterpret_cast<u32x2*>(region + l32 * COL_BYTES + (i * 32 + 8 * g + 4 * hi) * 2) = two;
+      }
+#pragma unroll
+    for (int q = lane; q < 32 * CHUNKS; q += 64) {
+      const int c = q / CHUNKS, part = q % CHUNKS;
+      // columns start at multiples of 8 bytes only: two 8-byte LDS reads per 16-byte global store
+      const u32x2 lo = *reinterpret_cast<const u32x2*>(region + c * COL_BYTES + part * 16);
+      const u32x2 up = *reinterpret_cast<const u32x2*>(region + c * COL_BYTES + part * 16 + 8);
+      const u32x4 v = {lo[0], lo[1], up[0], up[1]};
+      *reinterpret_cast<u32x4*>(ct + (size_t)(colw + j * 32 + c) * p.ct_rows + part * 8) = v;
     }
   }
 }
@@ -462,7 +522,16 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
       cur = nxt;
     }
   }
-  store_tile_h<TM, TN, EPI>(p, acc, m0 + wm0, n0 + wn0, l32, hi);
+  u16* stage = nullptr;
+  if (EPI != EPH_F32 && p.Ct) {
+    // every wavefront is done with the operand tiles (and all direct loads have landed): the LDS
+    // is free for the staging of the transposed output, one private region per wavefront
+    constexpr int REGION = 32 * (TM * 64 + 8);
+    static_assert((size_t)NW * REGION <= STAGES * (size_t)(BM + BN) * BK * sizeof(u16), "staging must fit the ring");
+    __syncthreads();
+    stage = smem_h + (size_t)wave * (REGION / 2);
+  }
+  store_tile_h<TM, TN, EPI>(p, acc, m0 + wm0, n0 + wn0, l32, hi, stage);
 }
 
 // Any-shape fallback: one thread per output element, fp32 accumulation in k order.
@@ -524,11 +593,17 @@ static hipError_t launch_dma(HGemmArgs& p, int batch, hipStream_t s) {
 }
 
 template <int EPI>
-static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant) {
+static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant, bool* wrote_ct) {
+  if (wrote_ct) *wrote_ct = p.Ct != nullptr && EPI != EPH_F32;
   if (p.M <= 0 || p.N <= 0 || batch <= 0) return hipSuccess;
   auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   const bool vec_ok = al16(p.A) && al16(p.B) && p.lda % 8 == 0 && p.ldb % 8 == 0 && p.batchA % 8 == 0 &&
                       p.batchB % 8 == 0 && p.K > 0;
+  // the transposed second output needs whole tiles inside one row group and 16-byte aligned stores
+  const bool want_ct = p.Ct != nullptr;
+  auto ct_ok = [&](int bm) {
+    return !want_ct || (p.ct_rows % bm == 0 && p.ct_rows % 8 == 0 && al16(p.Ct) && batch == 1);
+  };
   auto fits = [&](int bm, int bn, int bk) { return vec_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0; };
   if (variant == 0) {
     // 256 x 256 tiles with 8 wavefronts and direct-to-LDS loads once they cover the CUs (whole
@@ -540,6 +615,13 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     else if (fits(64, 64, 32)) variant = 5;
     else variant = -1;
   }
+  {  // the tile height decides whether the transposed output is possible; if not, drop it
+    const int bm = (variant == 3 || variant == 17) ? 128 : variant == 5 ? 64 : 256;
+    if (want_ct && (EPI == EPH_F32 || !ct_ok(bm))) {
+      p.Ct = nullptr;
+      if (wrote_ct) *wrote_ct = false;
+    }
+  }
   switch (variant) {
     case 3: if (fits(128, 128, 32)) return launch_h<128, 128, 32, 2, 2, EPI>(p, batch, s); break;
     case 4: if (fits(256, 256, 32)) return launch_h<256, 256, 32, 2, 4, EPI>(p, batch, s); break;
@@ -549,6 +631,8 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     case 19: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2>(p, batch, s); break;
     default: break;
   }
+  if (wrote_ct) *wrote_ct = false;  // the any-shape kernel has no transposed output
+  p.Ct = nullptr;
   launch_kernel((gemm_bf16_generic<EPI>), dim3((p.N + 15) / 16, (p.M + 15) / 16, batch), dim3(256), 0, s, p);
   return hipGetLastError();
 }
@@ -557,16 +641,18 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
 // 2 bf16 masked, 3 bf16 plain.
 hipError_t hgemm_nt(int batch, int M, int N, int K, const uint16_t* A, int lda, long long batchA, const uint16_t* B,
                     int ldb, long long batchB, void* C, int ldc, long long batchC, int out_kind, const float* bias,
-                    int relu, const uint16_t* mask, int ldmask, hipStream_t s, int variant) {
+                    int relu, const uint16_t* mask, int ldmask, hipStream_t s, int variant, uint16_t* Ct, int ct_rows,
+                    bool* wrote_ct) {
   HGemmArgs p{};
+  p.Ct = Ct; p.ct_rows = ct_rows;
   p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.batchA = batchA; p.batchB = batchB; p.batchC = batchC;
   p.bias = bias; p.relu = relu; p.mask = mask; p.ldmask = ldmask;
   switch (out_kind) {
-    case 0: return dispatch_h<EPH_F32>(p, batch, s, variant);
-    case 1: return dispatch_h<EPH_BIAS_RELU>(p, batch, s, variant);
-    case 2: return dispatch_h<EPH_MASK>(p, batch, s, variant);
-    default: return dispatch_h<EPH_BF16>(p, batch, s, variant);
+    case 0: return dispatch_h<EPH_F32>(p, batch, s, variant, wrote_ct);
+    case 1: return dispatch_h<EPH_BIAS_RELU>(p, batch, s, variant, wrote_ct);
+    case 2: return dispatch_h<EPH_MASK>(p, batch, s, variant, wrote_ct);
+    default: return dispatch_h<EPH_BF16>(p, batch, s, variant, wrote_ct);
   }
 }
 

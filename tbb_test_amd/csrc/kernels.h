@@ -58,10 +58,13 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
 
 // bf16: C = A[M,K] * B[N,K]^T with fp32 accumulation, both operands K-contiguous, blockIdx.z
 // batches with element strides batchA/B/C.  out_kind: 0 fp32 plain, 1 bf16 with bias + optional
-// ReLU, 2 bf16 zeroed where mask (bf16) <= 0, 3 bf16 plain.
+// ReLU, 2 bf16 zeroed where mask (bf16) <= 0, 3 bf16 plain.  Ct (bf16 output kinds, batch 1): the
+// result is also written transposed per group of ct_rows rows, Ct[row / ct_rows][col][row % ct_rows];
+// *wrote_ct tells whether the kernel that was chosen could do that (else the caller transposes).
 hipError_t hgemm_nt(int batch, int M, int N, int K, const uint16_t* A, int lda, long long batchA, const uint16_t* B,
                     int ldb, long long batchB, void* C, int ldc, long long batchC, int out_kind, const float* bias,
-                    int relu, const uint16_t* mask, int ldmask, hipStream_t s, int variant);
+                    int relu, const uint16_t* mask, int ldmask, hipStream_t s, int variant, uint16_t* Ct = nullptr,
+                    int ct_rows = 0, bool* wrote_ct = nullptr);
 // dst[z][c][r] = src[z][r][c] for 16-bit elements
 hipError_t transpose_bf16(int batch, int rows, int cols, const uint16_t* src, int ld_src, long long batch_src,
                           uint16_t* dst, int ld_dst, long long batch_dst, hipStream_t s);
