@@ -101,3 +101,48 @@ def test_bf16_config_5_full_size_sampled():
     want = oracle.reduce_sgd(Ws[l][ms].ravel(), np.stack([g.ravel() for g in grads]), LR).reshape(len(ms), -1)
     assert np.array_equal(W_new.view(np.uint32), want.view(np.uint32))
     h.close()
+
+
+@pytest.mark.parametrize("M,N,K,R", [(4096, 1024, 1024, 4), (4096, 4096, 4096, 2)])
+def test_gemm_size_independent_properties_at_full_size(M, N, K, R):
+    """Properties that need no oracle, at the GEMM shapes of configs 2 and 3, for the three raw
+    entry points: scaling an operand by a power of two scales the result bit for bit (no tile is
+    dropped, duplicated or mixed up), a second run gives the same bits, and the result of a
+    one-hot operand is the selected row / column of the other operand, exactly."""
+    rng = np.random.default_rng(M + N + K)
+    lib = capi.lib()
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)      # forward: X [M x K]
+    W = rng.uniform(-1, 1, (N, K)).astype(np.float32)      # W [N x K]
+    dZ = rng.standard_normal((M, N)).astype(np.float32)    # gradient [M x N]
+    dA, dW_, ddZ = (capi.DeviceBuffer.from_numpy(x) for x in (A, W, dZ))
+    dA2, ddZ2 = capi.DeviceBuffer.from_numpy(2 * A), capi.DeviceBuffer.from_numpy(2 * dZ)
+    out_y, out_dx, out_dw = capi.DeviceBuffer(M * N * 4), capi.DeviceBuffer(M * K * 4), capi.DeviceBuffer(R * N * K * 4)
+
+    def fwd(x):
+        capi.check(lib.mi_sgemm_nt(M, N, K, x.ptr, K, dW_.ptr, K, out_y.ptr, N, None, 0, None))
+        return out_y.to_numpy((M, N))
+
+    def dgrad(g):
+        capi.check(lib.mi_sgemm_nn(M, K, N, g.ptr, N, dW_.ptr, K, out_dx.ptr, K, None, 0, None))
+        return out_dx.to_numpy((M, K))
+
+    def wgrad(g):
+        capi.check(lib.mi_sgemm_tn(R, N, K, M // R, g.ptr, N, dA.ptr, K, out_dw.ptr, K, N * K, None, 0, None))
+        return out_dw.to_numpy((R, N, K))
+
+    for fn, one, two in ((fwd, dA, dA2), (dgrad, ddZ, ddZ2), (wgrad, ddZ, ddZ2)):
+        base = fn(one)
+        again = fn(one)
+        doubled = fn(two)
+        assert np.array_equal(base.view(np.uint32), again.view(np.uint32)), fn.__name__
+        assert np.array_equal((2 * base).view(np.uint32), doubled.view(np.uint32)), fn.__name__
+        assert np.isfinite(base).all() and np.abs(base).max() > 0
+
+    # one-hot rows of X pick columns of W^T: Y[i, :] = W[:, k_i]
+    picks = rng.integers(0, K, M)
+    onehot = np.zeros((M, K), np.float32)
+    onehot[np.arange(M), picks] = 1.0
+    d1 = capi.DeviceBuffer.from_numpy(onehot)
+    assert np.array_equal(fwd(d1), W[:, picks].T)
+    for b in (dA, dW_, ddZ, dA2, ddZ2, out_y, out_dx, out_dw, d1):
+        b.free()
