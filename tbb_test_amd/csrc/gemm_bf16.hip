@@ -653,13 +653,38 @@ hipError_t hgemm_nt(int batch, int M, int N, int K, const uint16_t* A, int lda, 
 }
 
 // ---- batched transpose: dst[z][c][r] = src[z][r][c], 16-bit elements, 64 x 64 tiles through LDS ----
+// VEC = true (tile-aligned shapes, 16-byte aligned rows on both sides): a thread moves 8 elements
+// with one 16-byte access on either side of the LDS tile; else element by element with bounds
+// checks.
+template <bool VEC>
 __global__ __launch_bounds__(256) void transpose16_kernel(u16* __restrict__ dst, const u16* __restrict__ src, int rows,
                                                           int cols, int ld_src, int ld_dst, long long batch_src,
                                                           long long batch_dst) {
-  __shared__ u16 tile[64][66];
+  __shared__ __attribute__((aligned(16))) u16 tile[64][72];  // 144-byte rows: 16-byte aligned, odd multiple of 16
   const u16* s = src + (size_t)blockIdx.z * batch_src;
   u16* d = dst + (size_t)blockIdx.z * batch_dst;
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  if (VEC) {
+    const int part = threadIdx.x & 7, line = threadIdx.x >> 3;  // 8 threads per 64-element row, 32 rows per pass
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = line + 32 * i;
+      *reinterpret_cast<u32x4*>(&tile[r][part * 8]) =
+          *reinterpret_cast<const u32x4*>(s + (size_t)(r0 + r) * ld_src + c0 + part * 8);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int c = line + 32 * i;  // output row = input column
+      u16 e[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) e[k] = tile[part * 8 + k][c];
+      const u32x4 v = {(unsigned)e[0] | ((unsigned)e[1] << 16), (unsigned)e[2] | ((unsigned)e[3] << 16),
+                       (unsigned)e[4] | ((unsigned)e[5] << 16), (unsigned)e[6] | ((unsigned)e[7] << 16)};
+      *reinterpret_cast<u32x4*>(d + (size_t)(c0 + c) * ld_dst + r0 + part * 8) = v;
+    }
+    return;
+  }
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   for (int i = ty; i < 64; i += 4) {
     const int r = r0 + i, c = c0 + tx;
@@ -675,20 +700,38 @@ __global__ __launch_bounds__(256) void transpose16_kernel(u16* __restrict__ dst,
 hipError_t transpose_bf16(int batch, int rows, int cols, const uint16_t* src, int ld_src, long long batch_src,
                           uint16_t* dst, int ld_dst, long long batch_dst, hipStream_t s) {
   if (batch <= 0 || rows <= 0 || cols <= 0) return hipSuccess;
-  launch_kernel(transpose16_kernel, dim3((cols + 63) / 64, (rows + 63) / 64, batch), dim3(256), 0, s, dst, src, rows,
-                     cols, ld_src, ld_dst, batch_src, batch_dst);
+  auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  const bool vec = rows % 64 == 0 && cols % 64 == 0 && ld_src % 8 == 0 && ld_dst % 8 == 0 && batch_src % 8 == 0 &&
+                   batch_dst % 8 == 0 && al16(src) && al16(dst);
+  const dim3 grid((cols + 63) / 64, (rows + 63) / 64, batch);
+  if (vec) launch_kernel(transpose16_kernel<true>, grid, dim3(256), 0, s, dst, src, rows, cols, ld_src, ld_dst, batch_src, batch_dst);
+  else launch_kernel(transpose16_kernel<false>, grid, dim3(256), 0, s, dst, src, rows, cols, ld_src, ld_dst, batch_src, batch_dst);
   return hipGetLastError();
 }
 
 // ---- row sums of a bf16 matrix in fp32: out[z*stride_out + r] = sum_c src[z][r][c] -------------------
-// One wavefront per row, lanes stride over the columns, fixed-order tree at the end.
+// One wavefront per row.  VEC = true (cols a multiple of 8, 16-byte aligned rows): a lane adds up
+// 8 consecutive elements per 16-byte load in element order, lanes stride over the row; else one
+// element per load.  Fixed-order tree over the lanes at the end.
+template <bool VEC>
 __global__ __launch_bounds__(256) void rowsum16_kernel(float* __restrict__ out, const u16* __restrict__ src, int rows,
                                                        int cols, int ld, long long batch_src, long long stride_out) {
   const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const u16* s = src + (size_t)blockIdx.y * batch_src + (size_t)row * ld;
   float v = 0.0f;
-  for (int c = lane; c < cols; c += 64) v += bf2f(s[c]);
+  if (VEC) {
+    for (int c = lane * 8; c < cols; c += 512) {
+      const u32x4 t = *reinterpret_cast<const u32x4*>(s + c);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        v += __uint_as_float(t[k] << 16);
+        v += __uint_as_float(t[k] & 0xffff0000u);
+      }
+    }
+  } else {
+    for (int c = lane; c < cols; c += 64) v += bf2f(s[c]);
+  }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
   if (lane == 0) out[(size_t)blockIdx.y * stride_out + row] = v;
@@ -697,8 +740,9 @@ __global__ __launch_bounds__(256) void rowsum16_kernel(float* __restrict__ out, 
 hipError_t rowsum_bf16(int batch, int rows, int cols, const uint16_t* src, int ld, long long batch_src, float* out,
                        long long stride_out, hipStream_t s) {
   if (batch <= 0 || rows <= 0) return hipSuccess;
-  launch_kernel(rowsum16_kernel, dim3((rows + 3) / 4, batch), dim3(256), 0, s, out, src, rows, cols, ld, batch_src,
-                     stride_out);
+  const bool vec = cols % 8 == 0 && ld % 8 == 0 && batch_src % 8 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+  if (vec) launch_kernel(rowsum16_kernel<true>, dim3((rows + 3) / 4, batch), dim3(256), 0, s, out, src, rows, cols, ld, batch_src, stride_out);
+  else launch_kernel(rowsum16_kernel<false>, dim3((rows + 3) / 4, batch), dim3(256), 0, s, out, src, rows, cols, ld, batch_src, stride_out);
   return hipGetLastError();
 }
 
