@@ -103,9 +103,12 @@ __device__ __forceinline__ void tile_of_workgroup(int id, int tiles_m, int tiles
 // pieces go through the LDS instead, one 32-column block at a time, columns padded by 8 bytes so
 // that the 32 lanes of a half-wave hit distinct banks, and are read back as 16-byte chunks: one
 // store instruction then writes whole runs of TM*64 contiguous bytes.
+// `mask_lds` != nullptr (EPH_MASK): the workgroup's mask tile lies in the LDS, row-major with
+// `mask_ld` elements per row; (row_l, col_l) is this wavefront's first row / column inside it.
 template <int TM, int TN, int EPI>
 __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[TM][TN], int row0, int colw, int l32,
-                                             int hi, u16* lds = nullptr) {
+                                             int hi, u16* lds = nullptr, const u16* mask_lds = nullptr, int mask_ld = 0,
+                                             int row_l = 0, int col_l = 0) {
   typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
   const int col0 = colw + l32;
   float bias_v[TN];
@@ -130,7 +133,9 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
             v += bias_v[j];
             if (p.relu) v = v > 0.0f ? v : 0.0f;
           } else if (EPI == EPH_MASK) {
-            if (!(bf2f(p.mask[(size_t)row * p.ldmask + col]) > 0.0f)) v = 0.0f;
+            const u16 mk = mask_lds ? mask_lds[(row - row0 + row_l) * mask_ld + col_l + l32 + j * 32]
+                                    : p.mask[(size_t)row * p.ldmask + col];
+            if (!(bf2f(mk) > 0.0f)) v = 0.0f;
           }
           const u16 o = f2bf(v);
           ch[(size_t)row * p.ldc + col] = o;
@@ -141,6 +146,7 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
     }
   }
   if (EPI == EPH_F32 || !p.Ct) return;
+  if (mask_lds && lds) __syncthreads();  // the staging regions overlap the mask tile other wavefronts still read
   // the tile lies inside one row group: ct_rows is a multiple of the tile height
   const int group = row0 / p.ct_rows, m_local0 = row0 - group * p.ct_rows;
   u16* __restrict__ ct = p.Ct + (size_t)group * p.N * p.ct_rows + m_local0;
@@ -519,15 +525,39 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
     }
   }
   u16* stage = nullptr;
+  const u16* mask_lds = nullptr;
+  bool synced = false;
+  if constexpr (EPI == EPH_MASK) {
+    // The ReLU mask is read at the output position: 2 bytes per lane and element straight from
+    // global memory are 64-byte pieces (measured +300 us on a 1.9 ms GEMM).  Bring the tile's
+    // mask into the idle LDS with direct loads (two 512-byte rows per instruction) instead.
+    constexpr int MASK_UNITS = BM * BN / 512;  // 1 KB pieces
+    static_assert((size_t)BM * BN <= STAGES * (size_t)(BM + BN) * BK, "the mask tile must fit the ring");
+    static_assert(BN * 2 % 16 == 0 && 1024 % (BN * 2) == 0 && MASK_UNITS % NW == 0, "mask tile shape");
+    if (p.ldmask % 8 == 0 && (reinterpret_cast<uintptr_t>(p.mask) & 15) == 0) {  // uniform
+      __syncthreads();  // every wavefront is done with the operand tiles
+      synced = true;
+      constexpr int CPR = BN / 8, RPU = 64 / CPR;  // 16-byte chunks per mask row, rows per piece
+#pragma unroll
+      for (int u = 0; u < MASK_UNITS / NW; ++u) {
+        const int unit = u * NW + wave;
+        const int row = unit * RPU + lane / CPR, c = lane % CPR;
+        load_to_lds(p.mask + (size_t)(m0 + row) * p.ldmask + n0 + c * 8, lds_base + 1024u * (unsigned)unit);
+      }
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+      __syncthreads();
+      mask_lds = smem_h;
+    }
+  }
   if (EPI != EPH_F32 && p.Ct) {
     // every wavefront is done with the operand tiles (and all direct loads have landed): the LDS
     // is free for the staging of the transposed output, one private region per wavefront
     constexpr int REGION = 32 * (TM * 64 + 8);
     static_assert((size_t)NW * REGION <= STAGES * (size_t)(BM + BN) * BK * sizeof(u16), "staging must fit the ring");
-    __syncthreads();
+    if (!synced) __syncthreads();
     stage = smem_h + (size_t)wave * (REGION / 2);
   }
-  store_tile_h<TM, TN, EPI>(p, acc, m0 + wm0, n0 + wn0, l32, hi, stage);
+  store_tile_h<TM, TN, EPI>(p, acc, m0 + wm0, n0 + wn0, l32, hi, stage, mask_lds, BN, wm0, wn0);
 }
 
 // Any-shape fallback: one thread per output element, fp32 accumulation in k order.
