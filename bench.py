@@ -167,7 +167,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.config}: {layers} FC layers of width {width}, ReLU between layers, "
                                f"batch {B} per replica x {R} replicas, lr {args.lr}, seed {args.seed}",
-                   "schedule": ("serial backward" if args.serial_backward else "weight-gradient GEMMs on a second stream")
+                   "schedule": ("serial backward" if args.serial_backward or args.config == "C5"
+                                else "weight-gradient GEMMs on a second stream")
                                + (", one update launch" if args.flat_update else ", per-layer update on the second stream"),
                    "device": info["name"], "num_cus": info["num_cus"]},
         "gemm_flop_per_step": gemm_flop_step,
