@@ -167,7 +167,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.config}: {layers} FC layers of width {width}, ReLU between layers, "
                                f"batch {B} per replica x {R} replicas, lr {args.lr}, seed {args.seed}",
-                   "schedule": ("serial backward" if args.serial_backward or args.config == "C5"
+                   "schedule": ("serial backward" if args.serial_backward or args.config in ("C3", "C5")
                                 else "weight-gradient GEMMs on a second stream")
                                + (", one update launch" if args.flat_update else ", per-layer update on the second stream"),
                    "device": info["name"], "num_cus": info["num_cus"]},

@@ -53,8 +53,8 @@ typedef enum mi_dtype {
 #define MI_FLAG_SERIAL_BACKWARD 0x8u /* keep the whole backward pass on one stream; default: the
                                     weight-gradient GEMMs run on a second stream next to the chain
                                     of input-gradient GEMMs (they are independent per layer),
-                                    except for large bf16 models, whose GEMMs fill the device
-                                    on their own */
+                                    except for models whose GEMMs have four or more 128 x 128
+                                    tiles per CU and fill the device on their own */
 
 /* Timing slots, same names and order as the reference's enum Breakdown
  * (mlp_bench_common.h:12-20). */
