@@ -751,6 +751,100 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
   write_tile<TM, TN, A_KMAJOR, B_KMAJOR, EPI, false>(p, C, acc, m0 + wm0, n0 + wn0, lane);
 }
 
+// ---- small problems: 32 x 32 tiles, K split over the four wavefronts of a workgroup --------------
+// With fewer 64 x 64 tiles than CUs (config 1: 512 x 512 outputs) the tiled kernels leave most
+// SIMDs idle and every wavefront walks the whole K on its own: 256 dependent 64-cycle MFMAs.  Here
+// a workgroup owns one 32 x 32 block of C and each of its four wavefronts (one per SIMD)
+// multiplies a quarter of K, so a 512 x 512 x 512 GEMM puts 64 MFMAs on each of the 1024 SIMDs.
+// The wavefronts share no operand data, so fragments are loaded from global memory straight into
+// the registers the MFMAs read -- no LDS tile, no barrier in the loop (the operands of such small
+// problems sit in the L2).  The four partial blocks are added through the LDS in wavefront order
+// (deterministic), wavefront w finishing rows 8w .. 8w+7 of the block.
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM>
+__global__ __launch_bounds__(256) void gemm_f32_splitk(GemmArgs p) {
+  __shared__ float part[4][16][64];
+  __shared__ float cs_part[4][32];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hi = lane >> 5;
+  const int tile_m = blockIdx.x / p.tiles_n, tile_n = blockIdx.x - tile_m * p.tiles_n;
+  const int m0 = tile_m * 32, n0 = tile_n * 32;
+  const float* __restrict__ A = p.A + (size_t)blockIdx.z * p.batchA;
+  const float* __restrict__ B = p.B + (size_t)blockIdx.z * p.batchB;
+  float* __restrict__ C = p.C + (size_t)blockIdx.z * p.batchC;
+  const int kq = p.K / 4, k_begin = wave * kq, chunks = kq / 8;
+  // lane (l32, hi) feeds MFMA step q of a chunk with k = chunk*8 + 4*hi + q
+  const float* a_ptr = A_KMAJOR ? A + (size_t)(m0 + l32) * p.lda + k_begin + 4 * hi
+                                : A + (size_t)(k_begin + 4 * hi) * p.lda + m0 + l32;
+  const float* b_ptr = B_KMAJOR ? B + (size_t)(n0 + l32) * p.ldb + k_begin + 4 * hi
+                                : B + (size_t)(k_begin + 4 * hi) * p.ldb + n0 + l32;
+  const size_t a_step = A_KMAJOR ? 8 : (size_t)8 * p.lda, b_step = B_KMAJOR ? 8 : (size_t)8 * p.ldb;
+  auto fetch = [](float (&f)[4], const float* ptr, int ld, bool kmajor) {
+    if (kmajor) {
+      const f32x4 t = *reinterpret_cast<const f32x4*>(ptr);
+      f[0] = t[0]; f[1] = t[1]; f[2] = t[2]; f[3] = t[3];
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) f[q] = ptr[(size_t)q * ld];
+    }
+  };
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+  const bool do_colsum = COLSUM && p.colsum != nullptr && tile_n == 0;
+  float cs = 0.0f;
+  constexpr int DEPTH = 4;  // chunks in flight
+  float fa[DEPTH][4], fb[DEPTH][4];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (d < chunks) {
+      fetch(fa[d], a_ptr + d * a_step, p.lda, A_KMAJOR);
+      fetch(fb[d], b_ptr + d * b_step, p.ldb, B_KMAJOR);
+    }
+  for (int c = 0; c < chunks; c += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (c + d >= chunks) break;
+      float ua[4], ub[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) { ua[q] = fa[d][q]; ub[q] = fb[d][q]; }
+      if (c + d + DEPTH < chunks) {
+        fetch(fa[d], a_ptr + (size_t)(c + d + DEPTH) * a_step, p.lda, A_KMAJOR);
+        fetch(fb[d], b_ptr + (size_t)(c + d + DEPTH) * b_step, p.ldb, B_KMAJOR);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ua[q], ub[q], acc, 0, 0, 0);
+        if (COLSUM && do_colsum) cs += ua[q];
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) part[wave][r][lane] = acc[r];
+  if (COLSUM && do_colsum) {
+    cs += __shfl_xor(cs, 32, 64);  // the two lane halves hold different k of the same column
+    if (hi == 0) cs_part[wave][l32] = cs;
+  }
+  __syncthreads();
+  if (COLSUM && do_colsum && tid < 32)
+    p.colsum[(size_t)blockIdx.z * p.batchColsum + m0 + tid] =
+        ((cs_part[0][tid] + cs_part[1][tid]) + cs_part[2][tid]) + cs_part[3][tid];
+  const int col = n0 + l32;
+  const float bias_v = (EPI == EPI_BIAS_RELU && p.bias) ? p.bias[col] : 0.0f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int r = 4 * wave + e;
+    float v = ((part[0][r][lane] + part[1][r][lane]) + part[2][r][lane]) + part[3][r][lane];
+    const int row = m0 + 8 * wave + 4 * hi + e;  // register r holds row 8*(r/4) + 4*hi + r%4
+    if (EPI == EPI_BIAS_RELU) {
+      v += bias_v;
+      if (p.relu) v = v > 0.0f ? v : 0.0f;
+    } else if (EPI == EPI_MASK) {
+      if (!(p.mask[(size_t)row * p.ldmask + col] > 0.0f)) v = 0.0f;
+    }
+    C[(size_t)row * p.ldc + col] = v;
+  }
+}
+
 // ---- any-shape fallback ----------------------------------------------------------------------
 // Plain LDS-tiled SIMT kernel with fully guarded loads and stores; used when a dimension is not
 // a multiple of the MFMA tile or a pointer / leading dimension is not 16-byte aligned.
@@ -856,6 +950,14 @@ static hipError_t launch_dma(GemmArgs& p, int batch, hipStream_t s) {
   return hipGetLastError();
 }
 
+template <bool AK, bool BKM, int EPI, bool COLSUM>
+static hipError_t launch_splitk(GemmArgs& p, int batch, hipStream_t s) {
+  p.tiles_m = p.M / 32;
+  p.tiles_n = p.N / 32;
+  launch_kernel((gemm_f32_splitk<AK, BKM, EPI, COLSUM>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0, s, p);
+  return hipGetLastError();
+}
+
 template <bool AK, bool BKM, int EPI>
 static hipError_t launch_generic(GemmArgs& p, int batch, hipStream_t s) {
   dim3 grid((p.N + 63) / 64, (p.M + 63) / 64, batch);
@@ -894,7 +996,8 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
     //   * an input-gradient GEMM that runs next to such a short-K weight gradient takes BK = 32:
     //     with 48 KB each, two weight-gradient workgroups would sit beside every input-gradient
     //     workgroup and slow the chain of dependent input-gradient GEMMs that bounds the step.
-    // Smaller problems fall back to 128 x 64 and 64 x 64 tiles to get enough workgroups.
+    // Smaller problems fall back to 128 x 64 and 64 x 64 tiles to get enough workgroups, the
+    // smallest (config 1) to the split-K kernel.
     const long long tiles128 = (long long)(p.M / 128) * (p.N / 128) * batch;
     constexpr bool kWeightGradient = !AK && !BKM;
     if (fits(128, 128, 32) && tiles128 >= 192 && ((kWeightGradient && p.K >= 512) || corun)) {
@@ -903,6 +1006,8 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
       variant = 33;
     } else if (fits(128, 64, 32) && tiles128 * 2 >= 192) {
       variant = 11;
+    } else if (fits(32, 32, 32) && (long long)(p.M / 64) * (p.N / 64) * batch < 192) {
+      variant = 50;  // fewer 64 x 64 tiles than CUs: 32 x 32 tiles with K split over the wavefronts
     } else if (fits(64, 64, 16)) {
       variant = 16;
     } else if (p.K > 0) {
@@ -931,6 +1036,7 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
     case 30: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 4>(p, batch, s); } break;
     case 31: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 33: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 50: if (fits(32, 32, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_splitk<AK, BKM, EPI, COLSUM>(p, batch, s); } break;
     default: break;
   }
   return launch_generic<AK, BKM, EPI>(p, batch, s);
