@@ -29,6 +29,7 @@
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "kernels.h"
 
@@ -562,9 +563,26 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
 // Timestamps taken inside the kernel show uniform K steps of 2 220-2 256 cycles against the 2 048
 // cycles of their 32 MFMAs per SIMD (BK = 16), 3 000 cycles before the first and 3 500 after the
 // last step.
-__device__ __forceinline__ void load_to_lds_f32(const float* src, unsigned lds_byte_addr) {
+__device__ __forceinline__ void load_to_lds_f32(const float* uniform_base, unsigned lane_byte_offset,
+                                                unsigned lds_byte_addr) {
   const unsigned lds_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr);
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory", "m0");
+  const unsigned long long b = reinterpret_cast<unsigned long long>(uniform_base);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b), hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+  const unsigned long long sbase = ((unsigned long long)hi << 32) | lo;
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(lane_byte_offset), "s"(sbase)
+               : "memory", "m0");
+}
+
+template <int... S, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, S...>, F&& f) {
+  (f(std::integral_constant<int, S>{}), ...);
+}
+// f(integral_constant<int, 0>), ..., f(integral_constant<int, N-1>)
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
 }
 
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
@@ -626,10 +644,11 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   float* __restrict__ C = p.C + (size_t)blockIdx.z * p.batchC;
 
-  // global source of this lane for each of its load instructions, and the advance per K step
-  const float* ga[NIA];
-  const float* gb[NIB];
-  auto sources = [&](auto& g, auto kmajor, auto rows_c, const float* op, int ld, int first_row, int ni) {
+  // Global source of the load instructions: a wave-uniform base pointer per operand (the tile's
+  // first element for the current K step, advanced with scalar adds) plus a constant 32-bit byte
+  // offset per lane and instruction -- no vector arithmetic in the K loop.
+  unsigned offa[NIA], offb[NIB];
+  auto offsets = [&](auto& off, auto kmajor, auto rows_c, int ld, int ni) {
     constexpr bool KM = decltype(kmajor)::value;
     constexpr int ROWS = decltype(rows_c)::value;
     for (int j = 0; j < ni; ++j) {
@@ -638,32 +657,30 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
         using ST = SwizzledTile<ROWS, BK>;
         constexpr int RPI = 64 / ST::kChunks;
         const int row = unit * RPI + lane / ST::kChunks, pc = lane % ST::kChunks;
-        g[j] = op + (size_t)(first_row + row) * ld + (pc ^ ST::swz(row)) * 4;
+        off[j] = 4u * ((unsigned)row * (unsigned)ld + (unsigned)(pc ^ ST::swz(row)) * 4u);
       } else {
         constexpr int CPR = ROWS / 4, KPI = 64 / CPR > 0 ? 64 / CPR : 1;
         static_assert(CPR <= 64, "a tile row must fit one load instruction");
         const int k = unit * KPI + lane / CPR, c = lane % CPR;
-        g[j] = op + (size_t)k * ld + first_row + c * 4;
+        off[j] = 4u * ((unsigned)k * (unsigned)ld + (unsigned)c * 4u);
       }
     }
   };
-  sources(ga, std::integral_constant<bool, A_KMAJOR>{}, std::integral_constant<int, BM>{},
-          p.A + (size_t)blockIdx.z * p.batchA, p.lda, m0, NIA);
-  sources(gb, std::integral_constant<bool, B_KMAJOR>{}, std::integral_constant<int, BN>{},
-          p.B + (size_t)blockIdx.z * p.batchB, p.ldb, n0, NIB);
+  offsets(offa, std::integral_constant<bool, A_KMAJOR>{}, std::integral_constant<int, BM>{}, p.lda, NIA);
+  offsets(offb, std::integral_constant<bool, B_KMAJOR>{}, std::integral_constant<int, BN>{}, p.ldb, NIB);
+  const float* a_base = p.A + (size_t)blockIdx.z * p.batchA + (A_KMAJOR ? (size_t)m0 * p.lda : (size_t)m0);
+  const float* b_base = p.B + (size_t)blockIdx.z * p.batchB + (B_KMAJOR ? (size_t)n0 * p.ldb : (size_t)n0);
   const size_t a_step = A_KMAJOR ? (size_t)BK : (size_t)BK * p.lda;
   const size_t b_step = B_KMAJOR ? (size_t)BK : (size_t)BK * p.ldb;
   auto issue = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < NIA; ++j) {
-      load_to_lds_f32(ga[j], lds_base + 4u * (unsigned)(buf * A_FLOATS + (j * NW + wave) * 256));
-      ga[j] += a_step;
-    }
+    for (int j = 0; j < NIA; ++j)
+      load_to_lds_f32(a_base, offa[j], lds_base + 4u * (unsigned)(buf * A_FLOATS + (j * NW + wave) * 256));
 #pragma unroll
-    for (int j = 0; j < NIB; ++j) {
-      load_to_lds_f32(gb[j], lds_base + 4u * (unsigned)(STAGES * A_FLOATS + buf * B_FLOATS + (j * NW + wave) * 256));
-      gb[j] += b_step;
-    }
+    for (int j = 0; j < NIB; ++j)
+      load_to_lds_f32(b_base, offb[j], lds_base + 4u * (unsigned)(STAGES * A_FLOATS + buf * B_FLOATS + (j * NW + wave) * 256));
+    a_base += a_step;
+    b_base += b_step;
   };
   auto frags = [&](float (&fa)[TM][4], float (&fb)[TN][4], int buf, int kk) {
     if constexpr (A_KMAJOR) load_frag_swz<BM, BK, TM>(fa, As(buf), wm0, kk, lane);
@@ -705,10 +722,13 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
 
   float fa[2][TM][4], fb[2][TN][4];
   frags(fa[0], fb[0], 0, 0);
-  int cur = 0;
-  for (int t = 0; t < nk; ++t) {
-    const int nxt = cur + 1 == STAGES ? 0 : cur + 1;
-    const int fill = cur == 0 ? STAGES - 1 : cur - 1;
+  // One K step at ring position `cur`.  The position is a compile-time constant (the loop below
+  // is unrolled over the ring) so that every LDS address of the step is a register plus an
+  // immediate offset.
+  auto step = [&](int t, auto cur_c) {
+    constexpr int cur = decltype(cur_c)::value;
+    constexpr int nxt = cur + 1 == STAGES ? 0 : cur + 1;
+    constexpr int fill = cur == 0 ? STAGES - 1 : cur - 1;
 #pragma unroll
     for (int kk = 0; kk < CH; ++kk) {
       const int fc = kk & 1, fn = fc ^ 1;
@@ -734,8 +754,14 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
         for (int k = 0; k < CS_ROWS; ++k) csum += col[k * BM];
       }
     }
-    cur = nxt;
-  }
+  };
+  int t = 0;
+  for (; t + STAGES <= nk; t += STAGES)
+    static_for<STAGES>([&](auto sc) { step(t + decltype(sc)::value, sc); });
+  // fewer than STAGES steps are left; the ring is back at position 0
+  static_for<STAGES - 1>([&](auto sc) {
+    if (t + decltype(sc)::value < nk) step(t + decltype(sc)::value, sc);
+  });
 
   if (COLSUM && do_colsum) {
     __syncthreads();  // every wavefront is done with the operand tiles: reuse LDS for the partials
