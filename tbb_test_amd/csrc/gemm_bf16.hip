@@ -22,6 +22,9 @@
 // conflicts); a lane fetches its 8 k values of one 32 x 32 block with one 16-byte LDS read.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+#include <utility>
+
 #include "kernels.h"
 
 namespace mi {
@@ -365,9 +368,24 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
 // Written this way the compiler does not track the load at all; the kernel waits on vmcnt itself
 // (its own waits can only become longer through the extra loads in flight, never shorter, because
 // vmcnt retires in order).  m0 carries the wave-uniform LDS byte address.
-__device__ __forceinline__ void load_to_lds(const u16* src, unsigned lds_byte_addr) {
+__device__ __forceinline__ void load_to_lds(const u16* uniform_base, unsigned lane_byte_offset, unsigned lds_byte_addr) {
   const unsigned lds_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr);
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory", "m0");
+  const unsigned long long b = reinterpret_cast<unsigned long long>(uniform_base);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b), hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+  const unsigned long long sbase = ((unsigned long long)hi << 32) | lo;
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(lane_byte_offset), "s"(sbase)
+               : "memory", "m0");
+}
+
+template <int... S, class F>
+__device__ __forceinline__ void static_for_h_impl(std::integer_sequence<int, S...>, F&& f) {
+  (f(std::integral_constant<int, S>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for_h(F&& f) {
+  static_for_h_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
 }
 
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
@@ -416,32 +434,35 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
   constexpr int ROWS_PER_LINE = 256 / (BK * 2) > 0 ? 256 / (BK * 2) : 1;
   auto swz = [](int row) { return (row / ROWS_PER_LINE) % VPR; };
 
-  // global source of this lane for each of its load instructions
+  // Global source of the load instructions: a wave-uniform base pointer per operand (the tile's
+  // first element for the current K step, advanced with scalar adds) plus a constant 32-bit byte
+  // offset per lane and instruction.  Together with the compile-time ring positions below this
+  // keeps vector arithmetic out of the K loop: VALU instructions share the issue port with the
+  // MFMAs, and a handful per step cost the fp32 kernel 4-6 %.
   const int lrow = lane / VPR, pc = lane % VPR;
-  const u16* ga[NIA];
-  const u16* gb[NIB];
+  unsigned offa[NIA], offb[NIB];
 #pragma unroll
   for (int j = 0; j < NIA; ++j) {
     const int row = (j * NW + wave) * RPI + lrow;
-    ga[j] = p.A + (size_t)blockIdx.z * p.batchA + (size_t)(m0 + row) * p.lda + (pc ^ swz(row)) * 8;
+    offa[j] = 2u * ((unsigned)row * (unsigned)p.lda + (unsigned)(pc ^ swz(row)) * 8u);
   }
 #pragma unroll
   for (int j = 0; j < NIB; ++j) {
     const int row = (j * NW + wave) * RPI + lrow;
-    gb[j] = p.B + (size_t)blockIdx.z * p.batchB + (size_t)(n0 + row) * p.ldb + (pc ^ swz(row)) * 8;
+    offb[j] = 2u * ((unsigned)row * (unsigned)p.ldb + (unsigned)(pc ^ swz(row)) * 8u);
   }
+  const u16* a_base = p.A + (size_t)blockIdx.z * p.batchA + (size_t)m0 * p.lda;
+  const u16* b_base = p.B + (size_t)blockIdx.z * p.batchB + (size_t)n0 * p.ldb;
   const unsigned lds_base = (unsigned)(size_t)((__attribute__((address_space(3))) const void*)smem_h);
   auto issue = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < NIA; ++j) {
-      load_to_lds(ga[j], lds_base + 2u * (unsigned)(buf * A_ELEMS + (j * NW + wave) * RPI * STRIDE));
-      ga[j] += BK;
-    }
+    for (int j = 0; j < NIA; ++j)
+      load_to_lds(a_base, offa[j], lds_base + 2u * (unsigned)(buf * A_ELEMS + (j * NW + wave) * RPI * STRIDE));
 #pragma unroll
-    for (int j = 0; j < NIB; ++j) {
-      load_to_lds(gb[j], lds_base + 2u * (unsigned)(STAGES * A_ELEMS + buf * B_ELEMS + (j * NW + wave) * RPI * STRIDE));
-      gb[j] += BK;
-    }
+    for (int j = 0; j < NIB; ++j)
+      load_to_lds(b_base, offb[j], lds_base + 2u * (unsigned)(STAGES * A_ELEMS + buf * B_ELEMS + (j * NW + wave) * RPI * STRIDE));
+    a_base += BK;
+    b_base += BK;
   };
   auto load_frags = [&](bf16x8 (&fa)[TM], bf16x8 (&fb)[TN], int buf, int kk) {
 #pragma unroll
@@ -481,8 +502,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
     if (nk > 0) issue(0);
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     ring_barrier();
-    for (int t = 0; t < nk; ++t) {
-      const int cur = t & 1;
+    // ring positions are compile-time constants (loop unrolled over the two buffers): every LDS
+    // address is a register plus an immediate
+    auto step2 = [&](int t, auto cur_c) {
+      constexpr int cur = decltype(cur_c)::value;
       if (t + 1 < nk) issue(cur ^ 1);
       load_frags(fa[0], fb[0], cur, 0);
 #pragma unroll
@@ -493,7 +516,13 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
       }
       __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
       ring_barrier();
+    };
+    int t = 0;
+    for (; t + 2 <= nk; t += 2) {
+      step2(t, std::integral_constant<int, 0>{});
+      step2(t + 1, std::integral_constant<int, 1>{});
     }
+    if (t < nk) step2(t, std::integral_constant<int, 0>{});
   } else {
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
@@ -503,10 +532,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
     ring_barrier();
 
     load_frags(fa[0], fb[0], 0, 0);
-    int cur = 0;
-    for (int t = 0; t < nk; ++t) {
-      const int nxt = cur + 1 == STAGES ? 0 : cur + 1;
-      const int fill = cur == 0 ? STAGES - 1 : cur - 1;
+    auto step = [&](int t, auto cur_c) {
+      constexpr int cur = decltype(cur_c)::value;
+      constexpr int nxt = cur + 1 == STAGES ? 0 : cur + 1;
+      constexpr int fill = cur == 0 ? STAGES - 1 : cur - 1;
 #pragma unroll
       for (int kk = 0; kk < CH; ++kk) {
         const int fc = kk & 1, fn = fc ^ 1;
@@ -521,8 +550,13 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
           if (t + STAGES - 1 < nk) issue(fill);
         }
       }
-      cur = nxt;
-    }
+    };
+    int t = 0;
+    for (; t + STAGES <= nk; t += STAGES)
+      static_for_h<STAGES>([&](auto sc) { step(t + decltype(sc)::value, sc); });
+    static_for_h<STAGES - 1>([&](auto sc) {
+      if (t + decltype(sc)::value < nk) step(t + decltype(sc)::value, sc);
+    });
   }
   u16* stage = nullptr;
   const u16* mask_lds = nullptr;
@@ -542,7 +576,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
       for (int u = 0; u < MASK_UNITS / NW; ++u) {
         const int unit = u * NW + wave;
         const int row = unit * RPU + lane / CPR, c = lane % CPR;
-        load_to_lds(p.mask + (size_t)(m0 + row) * p.ldmask + n0 + c * 8, lds_base + 1024u * (unsigned)unit);
+        load_to_lds(p.mask + (size_t)m0 * p.ldmask + n0, 2u * ((unsigned)row * (unsigned)p.ldmask + (unsigned)c * 8u),
+                    lds_base + 1024u * (unsigned)unit);
       }
       __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
       __syncthreads();
