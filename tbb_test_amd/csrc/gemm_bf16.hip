@@ -422,6 +422,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
   auto As = [&](int buf) { return smem_h + buf * A_ELEMS; };
   auto Bs = [&](int buf) { return smem_h + STAGES * A_ELEMS + buf * B_ELEMS; };
 
+  const unsigned lds_base = (unsigned)(size_t)((__attribute__((address_space(3))) const void*)smem_h);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hi = lane >> 5;
@@ -453,7 +454,6 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
   }
   const u16* a_base = p.A + (size_t)blockIdx.z * p.batchA + (size_t)m0 * p.lda;
   const u16* b_base = p.B + (size_t)blockIdx.z * p.batchB + (size_t)n0 * p.ldb;
-  const unsigned lds_base = (unsigned)(size_t)((__attribute__((address_space(3))) const void*)smem_h);
   auto issue = [&](int buf) {
 #pragma unroll
     for (int j = 0; j < NIA; ++j)
@@ -464,17 +464,29 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
     a_base += BK;
     b_base += BK;
   };
+  // LDS byte addresses of this lane's fragments for each 16-wide K chunk of a step (block 0 of
+  // the wavefront, ring buffer 0).  swz(row) is the same for all 32 x 32 blocks of a wavefront
+  // (they are 32 rows apart), so the other blocks and buffers are immediate offsets from these.
+  // The empty asm keeps the compiler from re-deriving them with vector adds inside the K loop.
+  static_assert(32 % (ROWS_PER_LINE * VPR) == 0, "the swizzle must repeat every 32 rows");
+  unsigned a_addr[CH], b_addr[CH];
+#pragma unroll
+  for (int kk = 0; kk < CH; ++kk) {
+    const int ra = wm0 + l32, rb = wn0 + l32;
+    a_addr[kk] = lds_base + 2u * (unsigned)(ra * STRIDE + ((kk * 2 + hi) ^ swz(ra)) * 8);
+    b_addr[kk] = lds_base + 2u * (unsigned)(STAGES * A_ELEMS + rb * STRIDE + ((kk * 2 + hi) ^ swz(rb)) * 8);
+    asm volatile("" : "+v"(a_addr[kk]), "+v"(b_addr[kk]));
+  }
+  typedef __attribute__((address_space(3))) const bf16x8 lds_frag;
   auto load_frags = [&](bf16x8 (&fa)[TM], bf16x8 (&fb)[TN], int buf, int kk) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int row = wm0 + i * 32 + l32;
-      fa[i] = *reinterpret_cast<const bf16x8*>(As(buf) + row * STRIDE + ((kk * 2 + hi) ^ swz(row)) * 8);
-    }
+    for (int i = 0; i < TM; ++i)
+      fa[i] = *reinterpret_cast<lds_frag*>((__attribute__((address_space(3))) const char*)(size_t)(
+          a_addr[kk] + 2u * (unsigned)(buf * A_ELEMS + i * 32 * STRIDE)));
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int row = wn0 + j * 32 + l32;
-      fb[j] = *reinterpret_cast<const bf16x8*>(Bs(buf) + row * STRIDE + ((kk * 2 + hi) ^ swz(row)) * 8);
-    }
+    for (int j = 0; j < TN; ++j)
+      fb[j] = *reinterpret_cast<lds_frag*>((__attribute__((address_space(3))) const char*)(size_t)(
+          b_addr[kk] + 2u * (unsigned)(buf * B_ELEMS + j * 32 * STRIDE)));
   };
 
   f32x16 acc[TM][TN];
