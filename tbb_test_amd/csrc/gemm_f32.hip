@@ -47,7 +47,7 @@ struct GemmArgs {
   const float* B;
   float* C;
   int lda, ldb, ldc;
-  // batch (blockIdx.z): element offsets added per batch index
+  // batch: element offsets added per batch index
   long long batchA, batchB, batchC;
   // epilogue
   const float* bias;  // EPI_BIAS_RELU: [N] or null
@@ -60,23 +60,27 @@ struct GemmArgs {
   // GUARD kernels: which 16-byte vector accesses the alignment of pointers and leading dimensions
   // allows (bit 0: A loads, bit 1: B loads, bit 2: C stores and mask loads)
   int vec_flags;
-  // tile rasterisation
-  int tiles_m, tiles_n;
+  // tile rasterisation (flat grid of tiles_m * tiles_n * batch workgroups)
+  int tiles_m, tiles_n, batch;
 };
 
-// Maps the flat workgroup index to a C tile.  Workgroups are handed to the 8 XCDs round-robin
-// (id % 8), each XCD has a private 4 MB L2, and about 32 workgroups (one per CU) of an XCD run at
-// the same time.
-//   * Large grids (tile counts divisible as needed): the grid is cut into super-tiles of 4 x 8
-//     tiles; XCD x owns super-tiles x, x+8, ... and walks each row by row, so the 32 tiles it
-//     runs together share 4 A panels and 8 B panels.
-//   * Otherwise, if the tile count is a multiple of 8: XCD x gets the contiguous range
-//     [x*T/8, (x+1)*T/8) of the row-major order (tiles of one row share their A panel).
+// Maps the flat workgroup index to a batch entry and a C tile.  Workgroups are handed to the 8
+// XCDs round-robin (id % 8), each XCD has a private 4 MB L2, and about 32 workgroups (one per CU)
+// of an XCD run at the same time.
+//   * Large grids (tile counts divisible as needed): the grid of one batch entry is cut into
+//     super-tiles of 4 x 8 tiles; XCD x owns super-tiles x, x+8, ... and walks each row by row, so
+//     the 32 tiles it runs together share 4 A panels and 8 B panels.
+//   * Otherwise, if the tile count of the whole batch is a multiple of 8: XCD x gets the contiguous
+//     range [x*T/8, (x+1)*T/8) of the (batch entry, row, column) order, so that the tiles it runs
+//     together belong to as few batch entries and rows as possible (tiles of one row share their
+//     A panel, tiles of one batch entry their B panels).
 //   * Otherwise the identity.
-__device__ __forceinline__ void tile_of_block(const GemmArgs& p, int& tm, int& tn) {
+__device__ __forceinline__ void tile_of_block(const GemmArgs& p, int& tm, int& tn, int& z) {
   int id = blockIdx.x;
   const int total = p.tiles_m * p.tiles_n;
   if ((p.tiles_m & 3) == 0 && (p.tiles_n & 7) == 0 && (total & 255) == 0 && total >= 512) {
+    z = id / total;  // total is a multiple of 8, so id % 8 is still the XCD
+    id -= z * total;
     const int xcd = id & 7, j = id >> 3;
     const int super = (j >> 5) * 8 + xcd, within = j & 31;
     const int super_cols = p.tiles_n >> 3;
@@ -84,10 +88,13 @@ __device__ __forceinline__ void tile_of_block(const GemmArgs& p, int& tm, int& t
     tn = (super % super_cols) * 8 + (within & 7);
     return;
   }
-  if ((total & 7) == 0) {
-    const int per_xcd = total >> 3;
+  const int all = total * p.batch;
+  if ((all & 7) == 0) {
+    const int per_xcd = all >> 3;
     id = (id & 7) * per_xcd + (id >> 3);
   }
+  z = id / total;
+  id -= z * total;
   tm = id / p.tiles_n;
   tn = id - tm * p.tiles_n;
 }
@@ -354,13 +361,13 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
   const int lane = tid & 63, wave = tid >> 6;
   const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
 
-  int tile_m, tile_n;
-  tile_of_block(p, tile_m, tile_n);
+  int tile_m, tile_n, bz;
+  tile_of_block(p, tile_m, tile_n, bz);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-  const float* __restrict__ A = p.A + (size_t)blockIdx.z * p.batchA;
-  const float* __restrict__ B = p.B + (size_t)blockIdx.z * p.batchB;
-  float* __restrict__ C = p.C + (size_t)blockIdx.z * p.batchC;
+  const float* __restrict__ A = p.A + (size_t)bz * p.batchA;
+  const float* __restrict__ B = p.B + (size_t)bz * p.batchB;
+  float* __restrict__ C = p.C + (size_t)bz * p.batchC;
 
   // first element of this workgroup's panel, and the pointer advance per K step
   const float* a_ptr = A_KMAJOR ? A + (size_t)m0 * p.lda : A + m0;
@@ -384,8 +391,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
   f32x4 ra[NVA], rb[NVB];
   const int nk = GUARD ? (p.K + BK - 1) / BK : p.K / BK;
   int kt = 0;  // index of the next K tile to request (GUARD loads address from scratch)
-  const float* __restrict__ a_op = p.A + (size_t)blockIdx.z * p.batchA;
-  const float* __restrict__ b_op = p.B + (size_t)blockIdx.z * p.batchB;
+  const float* __restrict__ a_op = p.A + (size_t)bz * p.batchA;
+  const float* __restrict__ b_op = p.B + (size_t)bz * p.batchB;
   auto mfma_chunk = [&](const float (&fa)[TM][4], const float (&fb)[TN][4]) {
 #pragma unroll
     for (int q = 0; q < 4; ++q)
@@ -526,7 +533,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
       float total = smem[tid];
 #pragma unroll
       for (int sl = 1; sl < CS_SLICES; ++sl) total += smem[sl * BM + tid];
-      if (!GUARD || m0 + tid < p.M) p.colsum[(size_t)blockIdx.z * p.batchColsum + m0 + tid] = total;
+      if (!GUARD || m0 + tid < p.M) p.colsum[(size_t)bz * p.batchColsum + m0 + tid] = total;
     }
   }
 
@@ -639,10 +646,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
 
-  int tile_m, tile_n;
-  tile_of_block(p, tile_m, tile_n);
+  int tile_m, tile_n, bz;
+  tile_of_block(p, tile_m, tile_n, bz);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  float* __restrict__ C = p.C + (size_t)blockIdx.z * p.batchC;
+  float* __restrict__ C = p.C + (size_t)bz * p.batchC;
 
   // Global source of the load instructions: a wave-uniform base pointer per operand (the tile's
   // first element for the current K step, advanced with scalar adds) plus a constant 32-bit byte
@@ -668,8 +675,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
   };
   offsets(offa, std::integral_constant<bool, A_KMAJOR>{}, std::integral_constant<int, BM>{}, p.lda, NIA);
   offsets(offb, std::integral_constant<bool, B_KMAJOR>{}, std::integral_constant<int, BN>{}, p.ldb, NIB);
-  const float* a_base = p.A + (size_t)blockIdx.z * p.batchA + (A_KMAJOR ? (size_t)m0 * p.lda : (size_t)m0);
-  const float* b_base = p.B + (size_t)blockIdx.z * p.batchB + (B_KMAJOR ? (size_t)n0 * p.ldb : (size_t)n0);
+  const float* a_base = p.A + (size_t)bz * p.batchA + (A_KMAJOR ? (size_t)m0 * p.lda : (size_t)m0);
+  const float* b_base = p.B + (size_t)bz * p.batchB + (B_KMAJOR ? (size_t)n0 * p.ldb : (size_t)n0);
   const size_t a_step = A_KMAJOR ? (size_t)BK : (size_t)BK * p.lda;
   const size_t b_step = B_KMAJOR ? (size_t)BK : (size_t)BK * p.ldb;
   auto issue = [&](int buf) {
@@ -771,7 +778,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
       float total = smem[tid];
 #pragma unroll
       for (int sl = 1; sl < CS_SLICES; ++sl) total += smem[sl * BM + tid];
-      p.colsum[(size_t)blockIdx.z * p.batchColsum + m0 + tid] = total;
+      p.colsum[(size_t)bz * p.batchColsum + m0 + tid] = total;
     }
   }
   write_tile<TM, TN, A_KMAJOR, B_KMAJOR, EPI, false>(p, C, acc, m0 + wm0, n0 + wn0, lane);
@@ -953,8 +960,8 @@ static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
   }
   p.tiles_m = GUARD ? (p.M + BM - 1) / BM : p.M / BM;
   p.tiles_n = GUARD ? (p.N + BN - 1) / BN : p.N / BN;
-  dim3 grid(p.tiles_m * p.tiles_n, 1, batch);
-  launch_kernel(kern, grid, dim3(WM * WN * 64), lds_bytes, s, p);
+  p.batch = batch;
+  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n * batch), dim3(WM * WN * 64), lds_bytes, s, p);
   return hipGetLastError();
 }
 
@@ -972,7 +979,8 @@ static hipError_t launch_dma(GemmArgs& p, int batch, hipStream_t s) {
   }
   p.tiles_m = p.M / BM;
   p.tiles_n = p.N / BN;
-  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
+  p.batch = batch;
+  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n * batch), dim3(WM * WN * 64), lds_bytes, s, p);
   return hipGetLastError();
 }
 
