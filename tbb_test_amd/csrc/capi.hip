@@ -440,7 +440,7 @@ int enqueue_step(mi_mlp* h, float lr) {
     explicit CorunScope(mi_mlp* h_) : h(h_) {}
     ~CorunScope() { h->corun = false; }
   } corun_scope(h);
-  const bool corun_cfg = !(h->flags & MI_FLAG_SERIAL_BACKWARD);
+  const bool corun_cfg = !(h->flags & MI_FLAG_SERIAL_BACKWARD) && !crowded;
   for (int l = h->L - 1; l >= 0; --l) {
     h->corun = corun_cfg && h->B < 512;
     if ((rc = op_wgrad(h, l, s2, true))) return rc;

@@ -419,9 +419,6 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
   static_assert(STAGES == 2 || (STAGES - 2) * INSTR <= 63, "vmcnt is a 6-bit counter");
 
   extern __shared__ __attribute__((aligned(16))) u16 smem_h[];
-  auto As = [&](int buf) { return smem_h + buf * A_ELEMS; };
-  auto Bs = [&](int buf) { return smem_h + STAGES * A_ELEMS + buf * B_ELEMS; };
-
   const unsigned lds_base = (unsigned)(size_t)((__attribute__((address_space(3))) const void*)smem_h);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -507,34 +504,52 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[fc][i], fb[fc][j], acc[i][j], 0, 0, 0);
   };
   if constexpr (STAGES == 2) {
-    // Two buffers (what fits when BK = 64 makes a 256 x 256 tile 64 KB): the loads of tile t+1 are
-    // issued at the top of step t into the buffer step t-1 read and have the whole step to land;
-    // one barrier at the step boundary.  BK = 64 rows are whole 128-byte lines, which the load path
-    // moves markedly faster than the half lines of BK = 32.
+    // Two buffers (what fits when BK = 64 makes a 256 x 256 tile 64 KB).  BK = 64 rows are whole
+    // 128-byte lines, which the load path moves markedly faster than the half lines of BK = 32.
+    // Step t multiplies buffer t % 2.  Before its last chunk every wavefront has issued all its
+    // reads of that buffer; it waits for them and for tile t+1 (the other buffer), then the
+    // barrier, then tile t+2 is requested into the buffer just read out and has a whole step to
+    // land.  The first fragments of tile t+1 are fetched during the last chunk's MFMAs, so no
+    // step starts with an empty MFMA pipe.
     if (nk > 0) issue(0);
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    if (nk > 1) {
+      issue(1);
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(INSTR));
+    } else {
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    }
     ring_barrier();
+    load_frags(fa[0], fb[0], 0, 0);
     // ring positions are compile-time constants (loop unrolled over the two buffers): every LDS
     // address is a register plus an immediate
-    auto step2 = [&](int t, auto cur_c) {
+    auto step2 = [&](int t, auto cur_c, auto steady_c) {
       constexpr int cur = decltype(cur_c)::value;
-      if (t + 1 < nk) issue(cur ^ 1);
-      load_frags(fa[0], fb[0], cur, 0);
+      constexpr bool steady = decltype(steady_c)::value;  // tile t+2 exists
 #pragma unroll
       for (int kk = 0; kk < CH; ++kk) {
         const int fc = kk & 1, fn = fc ^ 1;
         if (kk + 1 < CH) load_frags(fa[fn], fb[fn], cur, kk + 1);
+        else load_frags(fa[fn], fb[fn], cur ^ 1, 0);  // after the last tile: a harmless read of ring memory
         multiply(fc);
+        if (kk == CH - 2) {
+          // keeps this chunk's MFMAs above the barrier (it does not order register-only
+          // instructions, and an MFMA pipe that is empty at the barrier is lost time)
+          __builtin_amdgcn_sched_barrier(0);
+          __builtin_amdgcn_s_waitcnt(vmcnt_imm(0) & 0xc07f);  // vmcnt(0) and lgkmcnt(0)
+          ring_barrier();
+          if (steady || t + 2 < nk) issue(cur);
+        }
       }
-      __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-      ring_barrier();
     };
     int t = 0;
-    for (; t + 2 <= nk; t += 2) {
-      step2(t, std::integral_constant<int, 0>{});
-      step2(t + 1, std::integral_constant<int, 1>{});
+    for (; t + 4 <= nk; t += 2) {
+      step2(t, std::integral_constant<int, 0>{}, std::true_type{});
+      step2(t + 1, std::integral_constant<int, 1>{}, std::true_type{});
     }
-    if (t < nk) step2(t, std::integral_constant<int, 0>{});
+    static_for_h<3>([&](auto sc) {
+      constexpr int s = decltype(sc)::value;
+      if (t + s < nk) step2(t + s, std::integral_constant<int, s % 2>{}, std::false_type{});
+    });
   } else {
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
@@ -544,8 +559,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
     ring_barrier();
 
     load_frags(fa[0], fb[0], 0, 0);
-    auto step = [&](int t, auto cur_c) {
+    auto step = [&](int t, auto cur_c, auto steady_c) {
       constexpr int cur = decltype(cur_c)::value;
+      constexpr bool steady = decltype(steady_c)::value;  // tiles t+1 .. t+STAGES-1 all exist
       constexpr int nxt = cur + 1 == STAGES ? 0 : cur + 1;
       constexpr int fill = cur == 0 ? STAGES - 1 : cur - 1;
 #pragma unroll
@@ -555,19 +571,21 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
         else load_frags(fa[fn], fb[fn], nxt, 0);  // after the last tile: a harmless read of ring memory, keeps one code path
         multiply(fc);
         if (kk == CH - 2) {
+          __builtin_amdgcn_sched_barrier(0);  // this chunk's MFMAs stay above the barrier
           // tiles t+1 .. t+STAGES-2 are in flight; tile t+1 must have landed
-          if (t + STAGES - 2 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * INSTR));
+          if (steady || t + STAGES - 2 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * INSTR));
           else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
           ring_barrier();
-          if (t + STAGES - 1 < nk) issue(fill);
+          if (steady || t + STAGES - 1 < nk) issue(fill);
         }
       }
     };
     int t = 0;
-    for (; t + STAGES <= nk; t += STAGES)
-      static_for_h<STAGES>([&](auto sc) { step(t + decltype(sc)::value, sc); });
-    static_for_h<STAGES - 1>([&](auto sc) {
-      if (t + decltype(sc)::value < nk) step(t + decltype(sc)::value, sc);
+    for (; t + 2 * STAGES - 1 <= nk; t += STAGES)
+      static_for_h<STAGES>([&](auto sc) { step(t + decltype(sc)::value, sc, std::true_type{}); });
+    static_for_h<2 * STAGES - 2>([&](auto sc) {
+      constexpr int s = decltype(sc)::value;
+      if (t + s < nk) step(t + s, std::integral_constant<int, s % STAGES>{}, std::false_type{});
     });
   }
   u16* stage = nullptr;

@@ -732,8 +732,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
   // One K step at ring position `cur`.  The position is a compile-time constant (the loop below
   // is unrolled over the ring) so that every LDS address of the step is a register plus an
   // immediate offset.
-  auto step = [&](int t, auto cur_c) {
+  auto step = [&](int t, auto cur_c, auto steady_c) {
     constexpr int cur = decltype(cur_c)::value;
+    constexpr bool steady = decltype(steady_c)::value;  // tiles t+1 .. t+STAGES-1 all exist
     constexpr int nxt = cur + 1 == STAGES ? 0 : cur + 1;
     constexpr int fill = cur == 0 ? STAGES - 1 : cur - 1;
 #pragma unroll
@@ -749,11 +750,15 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
           for (int j = 0; j < TN; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[fc][i][q], fb[fc][j][q], acc[i][j], 0, 0, 0);
       if (kk == CH - 2) {
+        // The barrier does not order register-only instructions, and the scheduler otherwise sinks
+        // this chunk's MFMAs below it in some steps: the wavefronts then meet at the barrier with an
+        // empty MFMA pipe (measured: every such step 12 % longer).
+        __builtin_amdgcn_sched_barrier(0);
         // tiles t+1 .. t+STAGES-2 are in flight; tile t+1 must have landed
-        if (t + STAGES - 2 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_only((STAGES - 3) * INSTR));
+        if (steady || t + STAGES - 2 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_only((STAGES - 3) * INSTR));
         else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
         ring_barrier();
-        if (t + STAGES - 1 < nk) issue(fill);
+        if (steady || t + STAGES - 1 < nk) issue(fill);
       }
       if (kk == CH - 1 && COLSUM && do_colsum) {
         const float* col = As(cur) + (tid / BM) * CS_ROWS * BM + (tid % BM);
@@ -762,12 +767,15 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
       }
     }
   };
+  // Steady part: whole turns of the ring whose steps all refill a buffer -- straight-line code
+  // with no branch for the scheduler to stop at.
   int t = 0;
-  for (; t + STAGES <= nk; t += STAGES)
-    static_for<STAGES>([&](auto sc) { step(t + decltype(sc)::value, sc); });
-  // fewer than STAGES steps are left; the ring is back at position 0
-  static_for<STAGES - 1>([&](auto sc) {
-    if (t + decltype(sc)::value < nk) step(t + decltype(sc)::value, sc);
+  for (; t + 2 * STAGES - 1 <= nk; t += STAGES)
+    static_for<STAGES>([&](auto sc) { step(t + decltype(sc)::value, sc, std::true_type{}); });
+  // fewer than 2 * STAGES - 1 steps are left; the ring is back at position 0
+  static_for<2 * STAGES - 2>([&](auto sc) {
+    constexpr int s = decltype(sc)::value;
+    if (t + s < nk) step(t + s, std::integral_constant<int, s % STAGES>{}, std::false_type{});
   });
 
   if (COLSUM && do_colsum) {
@@ -965,22 +973,29 @@ static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
   return hipGetLastError();
 }
 
+// `exclusive`: ask for more than half of the CU's LDS, so that no second workgroup (of this or of
+// another kernel) shares the CU.  A workgroup of these kernels keeps the MFMA pipes of its CU busy
+// on its own; co-resident ones only interfere, and with several rounds of workgroups they make the
+// hardware's hand-out of workgroups to CUs uneven (measured on 1024 tiles: launches of 910 us and
+// of 1120 us at random with three 48 KB workgroups per CU, 910 us always with one).
 template <int BM, int BN, int BK, int WM, int WN, bool AK, bool BKM, int EPI, bool COLSUM, int STAGES>
-static hipError_t launch_dma(GemmArgs& p, int batch, hipStream_t s) {
+static hipError_t launch_dma(GemmArgs& p, int batch, hipStream_t s, bool exclusive = false) {
   constexpr size_t lds_bytes = STAGES * (size_t)(BM + BN) * BK * sizeof(float);
   static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB of LDS");
+  constexpr size_t kExclusiveBytes = 84 * 1024;
+  const size_t request = exclusive && lds_bytes < kExclusiveBytes ? kExclusiveBytes : lds_bytes;
   auto kern = gemm_f32_dma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES>;
-  static bool attr_set = false;
-  if (lds_bytes > 64 * 1024 && !attr_set) {
+  static size_t attr_bytes = 0;  // opt in to more than 64 KiB of dynamic LDS, per kernel
+  if (request > 64 * 1024 && request > attr_bytes) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)request);
     if (e != hipSuccess) return e;
-    attr_set = true;
+    attr_bytes = request;
   }
   p.tiles_m = p.M / BM;
   p.tiles_n = p.N / BN;
   p.batch = batch;
-  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n * batch), dim3(WM * WN * 64), lds_bytes, s, p);
+  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n * batch), dim3(WM * WN * 64), request, s, p);
   return hipGetLastError();
 }
 
@@ -1021,23 +1036,21 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
   if (corun) variant = 0;
   if (variant == 0) {
     // Automatic choice.  From about one 128 x 128 tile per CU on, the direct-to-LDS kernels with a
-    // ring of three buffers: BK = 16 (48 KB, up to three workgroups share a CU and one's prologue,
-    // epilogue and barrier waits are covered by another's MFMAs) or BK = 32 (96 KB, one workgroup
-    // per CU, half as many barriers).  Measured on the benchmark configurations, whole step:
-    //   * forward and input gradient: BK = 16;
-    //   * weight gradient (with its fused column sums): BK = 32 from K = 512 on, BK = 16 for the
-    //     short K of small per-replica batches;
-    //   * an input-gradient GEMM that runs next to such a short-K weight gradient takes BK = 32:
-    //     with 48 KB each, two weight-gradient workgroups would sit beside every input-gradient
-    //     workgroup and slow the chain of dependent input-gradient GEMMs that bounds the step.
+    // ring of three buffers.  Measured on the benchmark configurations, whole step:
+    //   * BK = 16 with the CU to itself (variant 34) everywhere, except
+    //   * a weight gradient with a short K (small per-replica batch: few K steps, so prologue and
+    //     epilogue weigh most) takes BK = 16 at its natural 48 KB and shares CUs (variant 33), and
+    //   * the input-gradient GEMM that runs next to such a weight gradient takes BK = 32 (96 KB,
+    //     variant 31): one weight-gradient workgroup fits beside it, not two, which would slow the
+    //     chain of dependent input-gradient GEMMs that bounds the step.
     // Smaller problems fall back to 128 x 64 and 64 x 64 tiles to get enough workgroups, the
     // smallest (config 1) to the split-K kernel.
     const long long tiles128 = (long long)(p.M / 128) * (p.N / 128) * batch;
     constexpr bool kWeightGradient = !AK && !BKM;
-    if (fits(128, 128, 32) && tiles128 >= 192 && ((kWeightGradient && p.K >= 512) || corun)) {
+    if (fits(128, 128, 32) && tiles128 >= 192 && corun) {
       variant = 31;
     } else if (fits(128, 128, 16) && tiles128 >= 192) {
-      variant = 33;
+      variant = kWeightGradient && p.K < 512 ? 33 : 34;
     } else if (fits(128, 64, 32) && tiles128 * 2 >= 192) {
       variant = 11;
     } else if (fits(32, 32, 32) && (long long)(p.M / 64) * (p.N / 64) * batch < 192) {
@@ -1070,6 +1083,7 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
     case 30: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 4>(p, batch, s); } break;
     case 31: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 33: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
+    case 34: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s, true); } break;
     case 50: if (fits(32, 32, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_splitk<AK, BKM, EPI, COLSUM>(p, batch, s); } break;
     default: break;
   }

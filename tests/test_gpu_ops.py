@@ -86,7 +86,7 @@ GEMM_SHAPES = [
     # ragged but 16-byte aligned storage: the guarded MFMA kernels
     (132, 260, 100), (1000, 520, 200), (36, 4, 64), (300, 128, 36), (128, 300, 4),
 ]
-VARIANTS = [0, 8, 9, 10, 11, 12, 15, 16, 17, 21, 22, 30, 31, 33, 50]
+VARIANTS = [0, 8, 9, 10, 11, 12, 15, 16, 17, 21, 22, 30, 31, 33, 34, 50]
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
