@@ -530,6 +530,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
         const int fc = kk & 1, fn = fc ^ 1;
         if (kk + 1 < CH) load_frags(fa[fn], fb[fn], cur, kk + 1);
         else load_frags(fa[fn], fb[fn], cur ^ 1, 0);  // after the last tile: a harmless read of ring memory
+        // The last reads of this buffer must have returned at the barrier below: issue them before
+        // this chunk's MFMAs, not (as the scheduler would) right in front of the wait.
+        if (kk == CH - 2) __builtin_amdgcn_sched_barrier(0);
         multiply(fc);
         if (kk == CH - 2) {
           // keeps this chunk's MFMAs above the barrier (it does not order register-only
