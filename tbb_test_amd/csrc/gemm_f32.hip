@@ -564,12 +564,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_mfma(GemmArgs p) {
 // through the extra loads in flight, never shorter: vmcnt retires in order).
 // The order of fragment reads and MFMAs inside a chunk is left to the compiler: pinning "reads of
 // the next chunk first" with sched_barrier was measured 2-4 % slower, interleaving reads between
-// MFMAs with sched_group_barrier within +-1 %.  Also measured without gain: issuing the loads
-// after the last chunk's MFMAs instead of right after the barrier, 128 x 64 tiles with two
-// workgroups per CU, 4 and 16 wavefronts per workgroup, non-temporal stores in the epilogue.
-// Timestamps taken inside the kernel show uniform K steps of 2 220-2 256 cycles against the 2 048
-// cycles of their 32 MFMAs per SIMD (BK = 16), 3 000 cycles before the first and 3 500 after the
-// last step.
+// MFMAs with sched_group_barrier within +-1 %.  The one pinned point is the fence in front of the
+// ring barrier (see the step below).  Also measured without gain: issuing the loads after the last
+// chunk's MFMAs instead of right after the barrier, rings of four and five buffers at BK = 16,
+// 128 x 64 tiles with two workgroups per CU, 4 and 16 wavefronts per workgroup, non-temporal
+// stores in the epilogue.  Timestamps taken inside the kernel: 1.3 us from the start of a
+// workgroup to its first tile in the LDS, 1.6 us from the last K step to the last store issued.
 __device__ __forceinline__ void load_to_lds_f32(const float* uniform_base, unsigned lane_byte_offset,
                                                 unsigned lds_byte_addr) {
   const unsigned lds_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr);
