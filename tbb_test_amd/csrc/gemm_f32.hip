@@ -62,41 +62,67 @@ struct GemmArgs {
   int vec_flags;
   // tile rasterisation (flat grid of tiles_m * tiles_n * batch workgroups)
   int tiles_m, tiles_n, batch;
+  int raster, per_xcd, total_shift, tiles_n_shift;  // see tile_of_block / set_raster
 };
 
 // Maps the flat workgroup index to a batch entry and a C tile.  Workgroups are handed to the 8
 // XCDs round-robin (id % 8), each XCD has a private 4 MB L2, and about 32 workgroups (one per CU)
 // of an XCD run at the same time.
-//   * Large grids (tile counts divisible as needed): the grid of one batch entry is cut into
-//     super-tiles of 4 x 8 tiles; XCD x owns super-tiles x, x+8, ... and walks each row by row, so
-//     the 32 tiles it runs together share 4 A panels and 8 B panels.
-//   * Otherwise, if the tile count of the whole batch is a multiple of 8: XCD x gets the contiguous
-//     range [x*T/8, (x+1)*T/8) of the (batch entry, row, column) order, so that the tiles it runs
-//     together belong to as few batch entries and rows as possible (tiles of one row share their
-//     A panel, tiles of one batch entry their B panels).
-//   * Otherwise the identity.
+//   * raster 2, large grids (tile counts divisible as needed): the grid of one batch entry is cut
+//     into super-tiles of 4 x 8 tiles; XCD x owns super-tiles x, x+8, ... and walks each row by
+//     row, so the 32 tiles it runs together share 4 A panels and 8 B panels.
+//   * raster 1, otherwise, if the tile count of the whole batch is a multiple of 8: XCD x gets the
+//     contiguous range [x*T/8, (x+1)*T/8) of the (batch entry, row, column) order, so that the
+//     tiles it runs together belong to as few batch entries and rows as possible (tiles of one row
+//     share their A panel, tiles of one batch entry their B panels).
+//   * raster 0, otherwise the identity.
+// The host chooses (set_raster) and passes the divisors' logarithms where they are powers of two:
+// every wavefront runs this before its first load, and an integer division is about 25 scalar
+// instructions.
+__device__ __forceinline__ int div_tiles(int x, int d, int shift) { return shift >= 0 ? x >> shift : x / d; }
+
 __device__ __forceinline__ void tile_of_block(const GemmArgs& p, int& tm, int& tn, int& z) {
   int id = blockIdx.x;
   const int total = p.tiles_m * p.tiles_n;
-  if ((p.tiles_m & 3) == 0 && (p.tiles_n & 7) == 0 && (total & 255) == 0 && total >= 512) {
-    z = id / total;  // total is a multiple of 8, so id % 8 is still the XCD
+  if (p.raster == 2) {
+    z = div_tiles(id, total, p.total_shift);  // total is a multiple of 8, so id % 8 is still the XCD
     id -= z * total;
     const int xcd = id & 7, j = id >> 3;
     const int super = (j >> 5) * 8 + xcd, within = j & 31;
     const int super_cols = p.tiles_n >> 3;
-    tm = (super / super_cols) * 4 + (within >> 3);
-    tn = (super % super_cols) * 8 + (within & 7);
+    const int sr = div_tiles(super, super_cols, p.tiles_n_shift >= 3 ? p.tiles_n_shift - 3 : -1);
+    tm = sr * 4 + (within >> 3);
+    tn = (super - sr * super_cols) * 8 + (within & 7);
     return;
   }
-  const int all = total * p.batch;
-  if ((all & 7) == 0) {
-    const int per_xcd = all >> 3;
-    id = (id & 7) * per_xcd + (id >> 3);
-  }
-  z = id / total;
+  if (p.raster == 1) id = (id & 7) * p.per_xcd + (id >> 3);
+  z = div_tiles(id, total, p.total_shift);
   id -= z * total;
-  tm = id / p.tiles_n;
+  tm = div_tiles(id, p.tiles_n, p.tiles_n_shift);
   tn = id - tm * p.tiles_n;
+}
+
+// Host side of tile_of_block; tiles_m and tiles_n are set.
+static inline int log2_if_pow2(int v) {
+  if (v <= 0 || (v & (v - 1)) != 0) return -1;
+  int s = 0;
+  while ((1 << s) < v) ++s;
+  return s;
+}
+static inline void set_raster(GemmArgs& p, int batch) {
+  const int total = p.tiles_m * p.tiles_n;
+  p.batch = batch;
+  p.total_shift = log2_if_pow2(total);
+  p.tiles_n_shift = log2_if_pow2(p.tiles_n);
+  p.per_xcd = 0;
+  if ((p.tiles_m & 3) == 0 && (p.tiles_n & 7) == 0 && (total & 255) == 0 && total >= 512) {
+    p.raster = 2;
+  } else if ((((long long)total * batch) & 7) == 0) {
+    p.raster = 1;
+    p.per_xcd = (int)(((long long)total * batch) >> 3);
+  } else {
+    p.raster = 0;
+  }
 }
 
 // Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does not wait for
@@ -968,7 +994,7 @@ static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
   }
   p.tiles_m = GUARD ? (p.M + BM - 1) / BM : p.M / BM;
   p.tiles_n = GUARD ? (p.N + BN - 1) / BN : p.N / BN;
-  p.batch = batch;
+  set_raster(p, batch);
   launch_kernel(kern, dim3(p.tiles_m * p.tiles_n * batch), dim3(WM * WN * 64), lds_bytes, s, p);
   return hipGetLastError();
 }
@@ -994,7 +1020,7 @@ static hipError_t launch_dma(GemmArgs& p, int batch, hipStream_t s, bool exclusi
   }
   p.tiles_m = p.M / BM;
   p.tiles_n = p.N / BN;
-  p.batch = batch;
+  set_raster(p, batch);
   launch_kernel(kern, dim3(p.tiles_m * p.tiles_n * batch), dim3(WM * WN * 64), request, s, p);
   return hipGetLastError();
 }
