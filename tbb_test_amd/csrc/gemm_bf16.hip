@@ -820,12 +820,20 @@ __global__ __launch_bounds__(256) void rowsum16_kernel(float* __restrict__ out, 
   const u16* s = src + (size_t)blockIdx.y * batch_src + (size_t)row * ld;
   float v = 0.0f;
   if (VEC) {
-    for (int c = lane * 8; c < cols; c += 512) {
-      const u32x4 t = *reinterpret_cast<const u32x4*>(s + c);
+    // four loads in flight per lane; the additions keep the element order of the plain loop
+    for (int c = lane * 8; c < cols; c += 4 * 512) {
+      u32x4 t[4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        v += __uint_as_float(t[k] << 16);
-        v += __uint_as_float(t[k] & 0xffff0000u);
+      for (int u = 0; u < 4; ++u)
+        if (c + u * 512 < cols) t[u] = *reinterpret_cast<const u32x4*>(s + c + u * 512);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (c + u * 512 >= cols) break;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          v += __uint_as_float(t[u][k] << 16);
+          v += __uint_as_float(t[u][k] & 0xffff0000u);
+        }
       }
     }
   } else {
