@@ -82,6 +82,9 @@ def run_tn(dZ, A, R, variant=0, with_colsum=True):
 GEMM_SHAPES = [
     (128, 128, 32), (256, 128, 64), (128, 256, 96), (512, 512, 512), (384, 640, 160),
     (64, 64, 32), (192, 64, 64),
+    # tile grids whose XCD-aware orders divide by something that is not a power of two:
+    # 8 x 3 tiles (contiguous range per XCD), 32 x 24 tiles (super-tiles, 3 per row)
+    (1024, 384, 64), (4096, 3072, 32),
     (1, 1, 1), (5, 3, 7), (100, 130, 50), (129, 127, 33), (257, 64, 1000), (64, 1, 64), (1, 300, 17),
     # ragged but 16-byte aligned storage: the guarded MFMA kernels
     (132, 260, 100), (1000, 520, 200), (36, 4, 64), (300, 128, 36), (128, 300, 4),
