@@ -218,3 +218,17 @@ def test_argument_errors_are_reported_not_fatal():
     # empty problems are fine
     assert lib.mi_sgemm_nt(0, 4, 4, None, 4, None, 4, None, 4, None, 0, None) == 0
     assert lib.mi_reduce_sgd_raw(None, None, 0, 0, 2, ctypes.c_float(0.1), None) == 0
+
+
+def test_k_zero_leaves_the_epilogue_of_an_all_zero_product():
+    """An empty contraction is a sum of nothing: C = relu(bias), 0 and 0 (cblas_sgemm with k = 0 and
+    beta = 0 writes zeros as well)."""
+    rng = np.random.default_rng(11)
+    M, N = 70, 130
+    b = _rand(rng, N)
+    got = run_nt(np.zeros((M, 0), np.float32), np.zeros((N, 0), np.float32), b, True)
+    assert np.array_equal(got, np.broadcast_to(np.maximum(b, 0.0), (M, N)))
+    got = run_nn(np.zeros((M, 0), np.float32), np.zeros((0, N), np.float32), None)
+    assert np.array_equal(got, np.zeros((M, N), np.float32))
+    C, S = run_tn(np.zeros((0, M), np.float32), np.zeros((0, N), np.float32), 2)
+    assert np.array_equal(C, np.zeros((2, M, N), np.float32)) and np.array_equal(S, np.zeros((2, M), np.float32))
