@@ -134,6 +134,21 @@ def main():
     finite = all(bool(np.isfinite(h.weight(l)).all()) for l in range(layers))
     h.close()
 
+    # What the matrix cores sustain right now with no memory traffic at all (register-resident
+    # MFMA loop, run on the warm device): context for the roofline fraction, which stays priced
+    # against the published peak.  The rate is power-limited and depends on the operand values;
+    # dense random operands draw more than the half-zero activations and gradients of the MLP, so
+    # the GEMMs of the step can come out above the random-operand figure.
+    def mfma_rate(operands):
+        import ctypes
+
+        r = ctypes.c_double()
+        capi.check(capi.lib().mi_probe_mfma_rate(1 if dtype == "bf16" else 0, operands, ctypes.byref(r), None))
+        return round(r.value, 1)
+    mfma_only = {"unit": "TFLOP/s", "random_operands": mfma_rate(2), "ones": mfma_rate(1), "zeros": mfma_rate(0),
+                 "how": "loop of independent MFMAs on register operands, no memory traffic, measured right "
+                        "after the steps above (mi_probe_mfma_rate)"}
+
     rows = R * B
     flop_per_gemm = 2.0 * rows * width * width          # every GEMM launch of a square model
     gemm_flop_step = 3 * layers * flop_per_gemm
@@ -181,7 +196,7 @@ def main():
                      "frac": round(gemm_tflops / peak, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get("gemm"),
                      "flop_per_launch": flop_per_gemm, "avg_launch_us": round(gemm_avg_ms * 1e3, 2),
-                     "launches": gemm_launches},
+                     "launches": gemm_launches, "mfma_only_rate": mfma_only},
         "roofline_reduce": {"kernel": "reduce_sgd_vec4", "bound": "hbm", "achieved": round(upd_gbps, 1),
                             "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(upd_gbps / PEAK_HBM_GBPS, 4),
                             "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get("reduce"),

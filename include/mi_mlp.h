@@ -170,6 +170,17 @@ int mi_rowsum_bf16(int batch, int rows, int cols, const void* src, int ld, long 
 /* Tuning hook for the bf16 kernel, like mi_set_gemm_variant. */
 int mi_set_hgemm_variant(int variant);
 
+/*
+ * Measurement aid without a counterpart in the reference: the rate, in TFLOP/s, of a loop of
+ * independent MFMAs on register operands (v_mfma_f32_32x32x2_f32 for MI_F32,
+ * v_mfma_f32_32x32x16_bf16 for MI_BF16) with no memory traffic, i.e. what the matrix cores of
+ * this device sustain at best.  operands: 0 = zeros, 1 = ones, 2 = pseudo-random values in
+ * [-1, 1) -- the rate is power-limited and depends on them.  Blocks until the measurement is
+ * done (about 0.2 s, best of many short batches, so that idle clocks do not enter); allocates and
+ * frees a small device buffer.
+ */
+int mi_probe_mfma_rate(int dtype, int operands, double* tflops, void* stream);
+
 /* fp32 <-> bf16 conversion of n contiguous elements on the device. */
 int mi_convert_f32_to_bf16(void* dst_bf16, const float* src, size_t n, void* stream);
 int mi_convert_bf16_to_f32(float* dst, const void* src_bf16, size_t n, void* stream);

@@ -50,6 +50,7 @@ SIGNATURES = {
     "mi_hgemm_tn": [c_int, c_int, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_int, c_longlong, c_void_p,
                     c_int, c_longlong, c_void_p],
     "mi_transpose_bf16": [c_int, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_int, c_longlong, c_void_p],
+    "mi_probe_mfma_rate": [c_int, c_int, POINTER(c_double), c_void_p],
     "mi_rowsum_bf16": [c_int, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_longlong, c_void_p],
     "mi_set_hgemm_variant": [c_int],
     "mi_convert_f32_to_bf16": [c_void_p, c_void_p, c_size_t, c_void_p],

@@ -701,6 +701,15 @@ int mi_set_hgemm_variant(int variant) {
   return MI_OK;
 }
 
+int mi_probe_mfma_rate(int dtype, int operands, double* tflops, void* stream) {
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "dtype must be MI_F32 or MI_BF16 (got %d)", dtype);
+  MI_REQUIRE(operands >= 0 && operands <= 2, "operands must be 0 (zeros), 1 (ones) or 2 (random), got %d", operands);
+  MI_REQUIRE(tflops != nullptr, "null result pointer");
+  hipError_t e = mi::probe_mfma_rate(dtype == MI_BF16, operands, tflops, as_stream(stream));
+  if (e != hipSuccess) return hip_fail(e, "mi_probe_mfma_rate");
+  return MI_OK;
+}
+
 int mi_convert_f32_to_bf16(void* dst, const float* src, size_t n, void* stream) {
   MI_REQUIRE(n == 0 || (dst && src), "null pointer");
   hipError_t e = mi::convert_f32_to_bf16((uint16_t*)dst, src, n, as_stream(stream));

@@ -66,6 +66,9 @@ hipError_t hgemm_nt(int batch, int M, int N, int K, const uint16_t* A, int lda, 
                     int relu, const uint16_t* mask, int ldmask, hipStream_t s, int variant, uint16_t* Ct = nullptr,
                     int ct_rows = 0, bool* wrote_ct = nullptr);
 // dst[z][c][r] = src[z][r][c] for 16-bit elements
+// mfma_probe.hip: TFLOP/s of a register-resident MFMA loop (operands: 0 zeros, 1 ones, 2 random)
+hipError_t probe_mfma_rate(bool bf16, int operands, double* tflops, hipStream_t s);
+
 hipError_t transpose_bf16(int batch, int rows, int cols, const uint16_t* src, int ld_src, long long batch_src,
                           uint16_t* dst, int ld_dst, long long batch_dst, hipStream_t s);
 // out[z*stride_out + r] = sum_c src[z][r][c] in fp32

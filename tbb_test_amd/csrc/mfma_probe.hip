@@ -1,0 +1,113 @@
+// Measurement aid: what do the MFMA pipes of this device sustain with nothing else going on?
+// A register-resident loop of independent MFMAs (four accumulator blocks per wavefront, four
+// wavefronts per SIMD), no memory traffic.  The rate depends on the operand values: the matrix
+// cores are power-limited, and constant operands toggle fewer wires than random mantissas.  The
+// GEMM kernels are priced against the published peak; this number says how much of the distance
+// to that peak is the device's and how much the kernels'.  No counterpart in the reference.
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+namespace mi {
+
+typedef float pf32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 pbf16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ unsigned probe_hash(unsigned x) {
+  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+  return x;
+}
+
+// operands: 0 zeros, 1 ones, 2 pseudo-random in [-1, 1), distinct per lane and register
+__device__ __forceinline__ float probe_value(int operands, unsigned h) {
+  return operands == 0 ? 0.0f : operands == 1 ? 1.0f : (float)(h & 0xffff) / 32768.0f - 1.0f;
+}
+
+__global__ __launch_bounds__(256) void mfma_rate_f32(float* out, int iters, int operands) {
+  pf32x16 acc[4];
+  for (int i = 0; i < 4; ++i)
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+  float a[8], b[8];
+  for (int i = 0; i < 8; ++i) {
+    const unsigned h = probe_hash(threadIdx.x * 16 + i + blockIdx.x * 7919);
+    a[i] = probe_value(operands, h);
+    b[i] = probe_value(operands, h >> 16);
+  }
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[(u + i) & 7], acc[i], 0, 0, 0);
+  }
+  float s = 0.0f;
+  for (int i = 0; i < 4; ++i)
+    for (int r = 0; r < 16; ++r) s += acc[i][r];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+__global__ __launch_bounds__(256) void mfma_rate_bf16(float* out, int iters, int operands) {
+  pf32x16 acc[4];
+  for (int i = 0; i < 4; ++i)
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+  pbf16x8 a[4], b[4];
+  for (int i = 0; i < 4; ++i)
+    for (int e = 0; e < 8; ++e) {
+      const unsigned h = probe_hash(threadIdx.x * 64 + i * 8 + e + blockIdx.x * 7919);
+      a[i][e] = (__bf16)probe_value(operands, h);
+      b[i][e] = (__bf16)probe_value(operands, h >> 16);
+    }
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[u], b[(u + i) & 3], acc[i], 0, 0, 0);
+  }
+  float s = 0.0f;
+  for (int i = 0; i < 4; ++i)
+    for (int r = 0; r < 16; ++r) s += acc[i][r];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+// Runs the loop on `s` in batches of three launches for about 0.2 s and returns the best batch in
+// TFLOP/s: the first tens of milliseconds after an idle period run at reduced clocks.
+hipError_t probe_mfma_rate(bool bf16, int operands, double* tflops, hipStream_t s) {
+  constexpr int kBlocks = 1024, kThreads = 256, kLaunches = 3;
+  const int iters = bf16 ? 8000 : 4000;
+  const int mfma_per_iter = bf16 ? 16 : 32;  // per wavefront
+  const double flop_per_mfma = bf16 ? 2.0 * 32 * 32 * 16 : 2.0 * 32 * 32 * 2;
+  const double flop_per_batch = (double)kBlocks * (kThreads / 64) * iters * mfma_per_iter * kLaunches * flop_per_mfma;
+  float* out = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipError_t e = hipMalloc((void**)&out, (size_t)kBlocks * kThreads * sizeof(float));
+  if (e != hipSuccess) return e;
+  double best = 0.0, total_ms = 0.0;
+  do {
+    if ((e = hipEventCreate(&e0)) != hipSuccess) break;
+    if ((e = hipEventCreate(&e1)) != hipSuccess) break;
+    for (int batch = 0; batch < 200 && total_ms < 200.0 && e == hipSuccess; ++batch) {
+      if ((e = hipEventRecord(e0, s)) != hipSuccess) break;
+      for (int w = 0; w < kLaunches; ++w) {
+        if (bf16) hipLaunchKernelGGL(mfma_rate_bf16, dim3(kBlocks), dim3(kThreads), 0, s, out, iters, operands);
+        else hipLaunchKernelGGL(mfma_rate_f32, dim3(kBlocks), dim3(kThreads), 0, s, out, iters, operands);
+      }
+      if ((e = hipEventRecord(e1, s)) != hipSuccess) break;
+      if ((e = hipEventSynchronize(e1)) != hipSuccess) break;
+      if ((e = hipGetLastError()) != hipSuccess) break;
+      float ms = 0.0f;
+      if ((e = hipEventElapsedTime(&ms, e0, e1)) != hipSuccess) break;
+      total_ms += ms;
+      const double rate = flop_per_batch / ((double)ms * 1e-3) / 1e12;
+      if (rate > best) best = rate;
+    }
+  } while (false);
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  (void)hipFree(out);
+  if (e != hipSuccess) return e;
+  *tflops = best;
+  return hipSuccess;
+}
+
+}  // namespace mi

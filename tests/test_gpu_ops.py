@@ -232,3 +232,16 @@ def test_k_zero_leaves_the_epilogue_of_an_all_zero_product():
     assert np.array_equal(got, np.zeros((M, N), np.float32))
     C, S = run_tn(np.zeros((0, M), np.float32), np.zeros((0, N), np.float32), 2)
     assert np.array_equal(C, np.zeros((2, M, N), np.float32)) and np.array_equal(S, np.zeros((2, M), np.float32))
+
+
+def test_mfma_rate_probe_reports_a_plausible_rate():
+    """The register-resident MFMA loop cannot beat the published peak by more than clock tolerance
+    and must come close to it: a rate far below would mean the probe measures something else."""
+    lib = capi.lib()
+    for dtype, peak in ((capi.MI_F32, 157.3), (capi.MI_BF16, 2516.6)):
+        for operands in (1, 2):
+            r = ctypes.c_double()
+            capi.check(lib.mi_probe_mfma_rate(dtype, operands, ctypes.byref(r), None))
+            assert 0.4 * peak < r.value < 1.1 * peak, (dtype, operands, r.value)
+    assert lib.mi_probe_mfma_rate(7, 1, ctypes.byref(r), None) == -1 and b"dtype" in lib.mi_last_error()
+    assert lib.mi_probe_mfma_rate(capi.MI_F32, 5, ctypes.byref(r), None) == -1
