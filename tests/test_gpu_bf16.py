@@ -142,12 +142,9 @@ STEP_CONFIGS = {
 }
 
 
-@pytest.mark.parametrize("name", list(STEP_CONFIGS))
-@pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, 0, capi.FLAG_PER_LAYER_UPDATE])
-def test_bf16_step_matches_fp32_oracle(name, flags):
-    nf, B, R = STEP_CONFIGS[name]
+def _check_bf16_step(nf, B, R, flags, seed=31):
     L = len(nf) - 1
-    X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed=31)
+    X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed=seed)
     rng = np.random.default_rng(1)
     bs = [(0.1 * rng.standard_normal(b.shape)).astype(np.float32) for b in bs]
     h = capi.MlpHandle(nf, B, R, dtype=capi.MI_BF16, flags=flags)
@@ -179,6 +176,26 @@ def test_bf16_step_matches_fp32_oracle(name, flags):
         assert rel_err(h.weight(l), ref.W_new[l]) <= BF16_TOL
         assert rel_err(h.bias(l), ref.b_new[l]) <= BF16_TOL
     h.close()
+
+
+@pytest.mark.parametrize("name", list(STEP_CONFIGS))
+@pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, 0, capi.FLAG_PER_LAYER_UPDATE])
+def test_bf16_step_matches_fp32_oracle(name, flags):
+    nf, B, R = STEP_CONFIGS[name]
+    _check_bf16_step(nf, B, R, flags)
+
+
+@pytest.mark.parametrize("variant", [13, 19])
+@pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, 0])
+def test_bf16_step_on_the_large_tile_kernels(variant, flags):
+    """The 256 x 256 direct-load kernels, which small models never pick by themselves: whole steps
+    with their fused transposed outputs and the ReLU mask tile brought into the LDS."""
+    lib = capi.lib()
+    capi.check(lib.mi_set_hgemm_variant(variant))
+    try:
+        _check_bf16_step([256, 512, 256, 512, 256], 128, 2, flags, seed=77)
+    finally:
+        lib.mi_set_hgemm_variant(0)
 
 
 def test_bf16_master_weights_stay_fp32():
