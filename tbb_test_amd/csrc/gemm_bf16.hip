@@ -108,7 +108,9 @@ __device__ __forceinline__ void tile_of_workgroup(int id, int tiles_m, int tiles
 // store instruction then writes whole runs of TM*64 contiguous bytes.
 // `mask_lds` != nullptr (EPH_MASK): the workgroup's mask tile lies in the LDS, row-major with
 // `mask_ld` elements per row; (row_l, col_l) is this wavefront's first row / column inside it.
-template <int TM, int TN, int EPI>
+// MASK_LDS is a template argument, not a test of mask_lds inside the loops: a pointer that may be
+// either LDS or global memory turns every mask read into a flat load behind a branch.
+template <int TM, int TN, int EPI, bool MASK_LDS = false>
 __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[TM][TN], int row0, int colw, int l32,
                                              int hi, u16* lds = nullptr, const u16* mask_lds = nullptr, int mask_ld = 0,
                                              int row_l = 0, int col_l = 0) {
@@ -120,36 +122,64 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
   float* __restrict__ cf = reinterpret_cast<float*>(p.C) + (size_t)blockIdx.z * p.batchC;
   u16* __restrict__ ch = reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC;
   unsigned pk[TM][TN][8];  // bf16 results, two rows per register: (4g, 4g+1) and (4g+2, 4g+3)
+  const unsigned mask_lds_addr = MASK_LDS ? (unsigned)(size_t)((__attribute__((address_space(3))) const void*)mask_lds) : 0u;
+  (void)mask_lds_addr;
+  if constexpr (EPI == EPH_F32) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = row0 + i * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
+      for (int r = 0; r < 16; ++r) {
+        const int row = row0 + i * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int col = col0 + j * 32;
-        float v = acc[i][j][r];
-        if (EPI == EPH_F32) {
-          cf[(size_t)row * p.ldc + col] = v;
-        } else {
+        for (int j = 0; j < TN; ++j) cf[(size_t)row * p.ldc + col0 + j * 32] = acc[i][j][r];
+      }
+    return;
+  } else {
+    // Two consecutive rows at a time: one v_cvt_pk_bf16_f32 rounds both (round to nearest even, the
+    // same result as the integer sequence of f2bf for finite values) and leaves them packed the way
+    // the transposed output wants them; the halves go out with 16-bit stores.
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int rp = 0; rp < 8; ++rp) {
+        const int row = row0 + i * 32 + 8 * (rp >> 1) + 4 * hi + 2 * (rp & 1);  // and row + 1
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int col = col0 + j * 32;
+          f32x2_t v = {acc[i][j][2 * rp], acc[i][j][2 * rp + 1]};
           if (EPI == EPH_BIAS_RELU) {
-            v += bias_v[j];
-            if (p.relu) v = v > 0.0f ? v : 0.0f;
+            v[0] += bias_v[j];
+            v[1] += bias_v[j];
+            if (p.relu) {
+              v[0] = v[0] > 0.0f ? v[0] : 0.0f;
+              v[1] = v[1] > 0.0f ? v[1] : 0.0f;
+            }
           } else if (EPI == EPH_MASK) {
-            const u16 mk = mask_lds ? mask_lds[(row - row0 + row_l) * mask_ld + col_l + l32 + j * 32]
-                                    : p.mask[(size_t)row * p.ldmask + col];
-            if (!(bf2f(mk) > 0.0f)) v = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              u16 mk;
+              if constexpr (MASK_LDS) {
+                typedef __attribute__((address_space(3))) const u16 lds_u16;
+                mk = reinterpret_cast<lds_u16*>(
+                    (__attribute__((address_space(3))) const char*)(size_t)mask_lds_addr)[(row + e - row0 + row_l) * mask_ld + col_l + l32 + j * 32];
+              } else {
+                mk = p.mask[(size_t)(row + e) * p.ldmask + col];
+              }
+              if (!(bf2f(mk) > 0.0f)) v[e] = 0.0f;
+            }
           }
-          const u16 o = f2bf(v);
-          ch[(size_t)row * p.ldc + col] = o;
-          if (r & 1) pk[i][j][r >> 1] |= (unsigned)o << 16;
-          else pk[i][j][r >> 1] = o;
+          const unsigned two = __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
+          pk[i][j][rp] = two;
+          ch[(size_t)row * p.ldc + col] = (u16)two;
+          ch[(size_t)(row + 1) * p.ldc + col] = (u16)(two >> 16);
         }
       }
     }
   }
   if (EPI == EPH_F32 || !p.Ct) return;
-  if (mask_lds && lds) __syncthreads();  // the staging regions overlap the mask tile other wavefronts still read
+  if (MASK_LDS && lds) __syncthreads();  // the staging regions overlap the mask tile other wavefronts still read
   // the tile lies inside one row group: ct_rows is a multiple of the tile height
   const int group = row0 / p.ct_rows, m_local0 = row0 - group * p.ct_rows;
   u16* __restrict__ ct = p.Ct + (size_t)group * p.N * p.ct_rows + m_local0;
@@ -626,7 +656,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
     if (!synced) __syncthreads();
     stage = smem_h + (size_t)wave * (REGION / 2);
   }
-  store_tile_h<TM, TN, EPI>(p, acc, m0 + wm0, n0 + wn0, l32, hi, stage, mask_lds, BN, wm0, wn0);
+  if (mask_lds) store_tile_h<TM, TN, EPI, true>(p, acc, m0 + wm0, n0 + wn0, l32, hi, stage, mask_lds, BN, wm0, wn0);
+  else store_tile_h<TM, TN, EPI, false>(p, acc, m0 + wm0, n0 + wn0, l32, hi, stage, nullptr, BN, wm0, wn0);
 }
 
 // Any-shape fallback: one thread per output element, fp32 accumulation in k order.
