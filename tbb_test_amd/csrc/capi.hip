@@ -420,9 +420,9 @@ int enqueue_step(mi_mlp* h, float lr) {
   // update launch: durations of kernels that overlap cannot be attributed to a kernel.
   const bool per_layer = (h->flags & MI_FLAG_PER_LAYER_UPDATE) != 0 && !h->timing;
   // Two backward streams pay while a GEMM launch leaves CUs idle at its start and end, i.e. up to
-  // a few tiles per CU (configs 2 and 4: 256 tiles of 128 x 128 per input-gradient launch, 6-7 %
+  // a few tiles per CU (configs 2 and 4: 256 tiles of 128 x 128 per input-gradient launch, 3-5 %
   // faster with two streams).  GEMMs with many tiles per CU only get in each other's way (config
-  // 3, 1024 tiles: 12.14 ms with one backward stream, 12.31 ms with two; config 5: 49.4 / 50.8 ms).
+  // 3, 1024 tiles: 11.32 ms with one backward stream, 11.47 ms with two; config 5: 45.9 / 47.1 ms).
   const bool crowded = (long long)(h->MB / 128) * (long long)(h->maxw() / 128) >= 1024;
   const bool dual = !(h->flags & MI_FLAG_SERIAL_BACKWARD) && !h->timing && !crowded;
   hipStream_t s2 = dual ? h->stream2 : s;
