@@ -51,6 +51,11 @@ METRIC = "MLP fwd+bwd+reduce step ms & TFLOP/s on 1 MI355X; grad-reduce GB/s"
 # input-gradient launches.  None = not measured for that configuration.
 MEASURED_TRAFFIC_BYTES = {
     "C2": {"gemm": (50.4e6 + 16.8e6 + 50.4e6 + 16.8e6 + 67.2e6 + 16.8e6) / 3, "reduce": 167.8e6 + 33.6e6},
+    # configs 3-5: mean over the GEMM launches of a step (forward, weight gradient, input gradient
+    # with and without mask, weighted by their counts)
+    "C3": {"gemm": 911.7e6, "reduce": 805.5e6 + 268.5e6},
+    "C4": {"gemm": 189.3e6, "reduce": 3021.4e6 + 335.7e6},
+    "C5": {"gemm": 4010.5e6, "reduce": 10738.7e6 + 3221.6e6},
 }
 
 
