@@ -52,7 +52,10 @@ def test_bf16_helpers_round_to_nearest_even():
 
 
 HSHAPES = [(64, 64, 32), (128, 128, 64), (256, 256, 96), (512, 256, 128), (256, 512, 32), (7, 5, 9), (100, 130, 50),
-           (129, 64, 40), (256, 256, 512)]
+           (129, 64, 40), (256, 256, 512),
+           # K loops of the direct-load kernels: one step, and every length of the conditional tail after
+           # the branch-free turns of the ring (two buffers at BK = 64, four at BK = 32)
+           (256, 256, 64), (256, 256, 192), (256, 256, 320), (256, 256, 448)]
 HVARIANTS = [0, 3, 4, 5, 13, 17, 19]
 
 
