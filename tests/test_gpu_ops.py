@@ -85,6 +85,8 @@ GEMM_SHAPES = [
     # tile grids whose XCD-aware orders divide by something that is not a power of two:
     # 8 x 3 tiles (contiguous range per XCD), 32 x 24 tiles (super-tiles, 3 per row)
     (1024, 384, 64), (4096, 3072, 32),
+    # K loops of the direct-load kernels: a single step, and the longest conditional tail of a ring of four
+    (128, 128, 16), (128, 128, 320),
     (1, 1, 1), (5, 3, 7), (100, 130, 50), (129, 127, 33), (257, 64, 1000), (64, 1, 64), (1, 300, 17),
     # ragged but 16-byte aligned storage: the guarded MFMA kernels
     (132, 260, 100), (1000, 520, 200), (36, 4, 64), (300, 128, 36), (128, 300, 4),
