@@ -432,6 +432,8 @@ __device__ __forceinline__ void ring_barrier() {
   asm volatile("" ::: "memory");
 }
 
+// The lambdas are always_inline: left to its cost model the compiler keeps the K-step lambdas of
+// large instantiations as real functions, and the accumulators they capture then live in memory.
 template <int BM, int BN, int BK, int WM, int WN, int EPI, int STAGES>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
   constexpr int NW = WM * WN;
@@ -482,7 +484,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
   }
   const u16* a_base = p.A + (size_t)blockIdx.z * p.batchA + (size_t)m0 * p.lda;
   const u16* b_base = p.B + (size_t)blockIdx.z * p.batchB + (size_t)n0 * p.ldb;
-  auto issue = [&](int buf) {
+  auto issue = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < NIA; ++j)
       load_to_lds(a_base, offa[j], lds_base + 2u * (unsigned)(buf * A_ELEMS + (j * NW + wave) * RPI * STRIDE));
@@ -527,7 +529,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
 
   const int nk = p.K / BK;
   bf16x8 fa[2][TM], fb[2][TN];
-  auto multiply = [&](int fc) {
+  auto multiply = [&](int fc) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -553,7 +555,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
     load_frags(fa[0], fb[0], 0, 0);
     // ring positions are compile-time constants (loop unrolled over the two buffers): every LDS
     // address is a register plus an immediate
-    auto step2 = [&](int t, auto cur_c, auto steady_c) {
+    auto step2 = [&](int t, auto cur_c, auto steady_c) __attribute__((always_inline)) {
       constexpr int cur = decltype(cur_c)::value;
       constexpr bool steady = decltype(steady_c)::value;  // tile t+2 exists
 #pragma unroll
@@ -593,7 +595,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
     ring_barrier();
 
     load_frags(fa[0], fb[0], 0, 0);
-    auto step = [&](int t, auto cur_c, auto steady_c) {
+    auto step = [&](int t, auto cur_c, auto steady_c) __attribute__((always_inline)) {
       constexpr int cur = decltype(cur_c)::value;
       constexpr bool steady = decltype(steady_c)::value;  // tiles t+1 .. t+STAGES-1 all exist
       constexpr int nxt = cur + 1 == STAGES ? 0 : cur + 1;
