@@ -141,9 +141,8 @@ def main():
 
     # What the matrix cores sustain right now with no memory traffic at all (register-resident
     # MFMA loop, run on the warm device): context for the roofline fraction, which stays priced
-    # against the published peak.  The rate is power-limited and depends on the operand values;
-    # dense random operands draw more than the half-zero activations and gradients of the MLP, so
-    # the GEMMs of the step can come out above the random-operand figure.
+    # against the published peak.  The bf16 rate is power-limited and depends on the operand
+    # values (dense random operands draw more than constant ones); the fp32 rate does not.
     def mfma_rate(operands):
         import ctypes
 

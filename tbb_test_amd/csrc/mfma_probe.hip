@@ -1,5 +1,5 @@
 // Measurement aid: what do the MFMA pipes of this device sustain with nothing else going on?
-// A register-resident loop of independent MFMAs (four accumulator blocks per wavefront, four
+// A register-resident loop of independent MFMAs (four accumulator blocks per wavefront, up to four
 // wavefronts per SIMD), no memory traffic.  The rate depends on the operand values: the matrix
 // cores are power-limited, and constant operands toggle fewer wires than random mantissas.  The
 // GEMM kernels are priced against the published peak; this number says how much of the distance
@@ -70,27 +70,41 @@ __global__ __launch_bounds__(256) void mfma_rate_bf16(float* out, int iters, int
   out[blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
-// Runs the loop on `s` in batches of three launches for about 0.2 s and returns the best batch in
-// TFLOP/s: the first tens of milliseconds after an idle period run at reduced clocks.
+// Runs the loop on `s` in batches of three launches for about 0.4 s and returns the average rate
+// of the second half in TFLOP/s (the first tens of milliseconds after an idle period run at
+// reduced clocks).  The grid is exactly what is resident at once, four workgroups per CU or fewer
+// if the register count allows fewer: a grid that needs a second, partly filled round would
+// measure that tail, not the MFMA pipes.
 hipError_t probe_mfma_rate(bool bf16, int operands, double* tflops, hipStream_t s) {
-  constexpr int kBlocks = 1024, kThreads = 256, kLaunches = 3;
+  constexpr int kThreads = 256, kLaunches = 3;
   const int iters = bf16 ? 8000 : 4000;
   const int mfma_per_iter = bf16 ? 16 : 32;  // per wavefront
   const double flop_per_mfma = bf16 ? 2.0 * 32 * 32 * 16 : 2.0 * 32 * 32 * 2;
-  const double flop_per_batch = (double)kBlocks * (kThreads / 64) * iters * mfma_per_iter * kLaunches * flop_per_mfma;
+  int dev = 0, cus = 0, per_cu = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e == hipSuccess)
+    e = bf16 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, mfma_rate_bf16, kThreads, 0)
+             : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, mfma_rate_f32, kThreads, 0);
+  if (e != hipSuccess) return e;
+  if (per_cu > 4) per_cu = 4;
+  if (per_cu < 1 || cus < 1) return hipErrorInvalidValue;
+  const int blocks = cus * per_cu;
+  const double flop_per_batch = (double)blocks * (kThreads / 64) * iters * mfma_per_iter * kLaunches * flop_per_mfma;
   float* out = nullptr;
   hipEvent_t e0 = nullptr, e1 = nullptr;
-  hipError_t e = hipMalloc((void**)&out, (size_t)kBlocks * kThreads * sizeof(float));
+  e = hipMalloc((void**)&out, (size_t)blocks * kThreads * sizeof(float));
   if (e != hipSuccess) return e;
-  double best = 0.0, total_ms = 0.0;
+  double total_ms = 0.0, late_ms = 0.0;
+  int late_batches = 0;
   do {
     if ((e = hipEventCreate(&e0)) != hipSuccess) break;
     if ((e = hipEventCreate(&e1)) != hipSuccess) break;
-    for (int batch = 0; batch < 200 && total_ms < 200.0 && e == hipSuccess; ++batch) {
+    for (int batch = 0; batch < 400 && total_ms < 400.0 && e == hipSuccess; ++batch) {
       if ((e = hipEventRecord(e0, s)) != hipSuccess) break;
       for (int w = 0; w < kLaunches; ++w) {
-        if (bf16) hipLaunchKernelGGL(mfma_rate_bf16, dim3(kBlocks), dim3(kThreads), 0, s, out, iters, operands);
-        else hipLaunchKernelGGL(mfma_rate_f32, dim3(kBlocks), dim3(kThreads), 0, s, out, iters, operands);
+        if (bf16) hipLaunchKernelGGL(mfma_rate_bf16, dim3(blocks), dim3(kThreads), 0, s, out, iters, operands);
+        else hipLaunchKernelGGL(mfma_rate_f32, dim3(blocks), dim3(kThreads), 0, s, out, iters, operands);
       }
       if ((e = hipEventRecord(e1, s)) != hipSuccess) break;
       if ((e = hipEventSynchronize(e1)) != hipSuccess) break;
@@ -98,15 +112,18 @@ hipError_t probe_mfma_rate(bool bf16, int operands, double* tflops, hipStream_t 
       float ms = 0.0f;
       if ((e = hipEventElapsedTime(&ms, e0, e1)) != hipSuccess) break;
       total_ms += ms;
-      const double rate = flop_per_batch / ((double)ms * 1e-3) / 1e12;
-      if (rate > best) best = rate;
+      if (total_ms > 200.0) {
+        late_ms += ms;
+        ++late_batches;
+      }
     }
   } while (false);
   if (e0) (void)hipEventDestroy(e0);
   if (e1) (void)hipEventDestroy(e1);
   (void)hipFree(out);
   if (e != hipSuccess) return e;
-  *tflops = best;
+  if (late_batches == 0 || late_ms <= 0.0) return hipErrorUnknown;
+  *tflops = flop_per_batch * late_batches / (late_ms * 1e-3) / 1e12;
   return hipSuccess;
 }
 
