@@ -175,7 +175,7 @@ int mi_set_hgemm_variant(int variant);
  * independent MFMAs on register operands (v_mfma_f32_32x32x2_f32 for MI_F32,
  * v_mfma_f32_32x32x16_bf16 for MI_BF16) with no memory traffic, i.e. what the matrix cores of
  * this device sustain at best.  operands: 0 = zeros, 1 = ones, 2 = pseudo-random values in
- * [-1, 1) -- the rate is power-limited and depends on them.  Blocks until the measurement is
+ * [-1, 1) -- the bf16 rate is power-limited and depends on them.  Blocks until the measurement is
  * done (about 0.4 s; the rate is the average over the second half, so that idle clocks do not
  * enter); allocates and frees a small device buffer.
  */

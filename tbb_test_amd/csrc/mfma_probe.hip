@@ -1,7 +1,8 @@
 // Measurement aid: what do the MFMA pipes of this device sustain with nothing else going on?
 // A register-resident loop of independent MFMAs (four accumulator blocks per wavefront, up to four
-// wavefronts per SIMD), no memory traffic.  The rate depends on the operand values: the matrix
-// cores are power-limited, and constant operands toggle fewer wires than random mantissas.  The
+// wavefronts per SIMD), no memory traffic.  For bf16 the rate depends on the operand values (the
+// matrix cores are power-limited there, and constant operands toggle fewer wires than random
+// mantissas: 2 380 against 1 780 TFLOP/s measured); for fp32 it does not (155 TFLOP/s).  The
 // GEMM kernels are priced against the published peak; this number says how much of the distance
 // to that peak is the device's and how much the kernels'.  No counterpart in the reference.
 #include <hip/hip_runtime.h>
