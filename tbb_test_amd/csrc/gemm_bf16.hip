@@ -484,15 +484,24 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
   }
   const u16* a_base = p.A + (size_t)blockIdx.z * p.batchA + (size_t)m0 * p.lda;
   const u16* b_base = p.B + (size_t)blockIdx.z * p.batchB + (size_t)n0 * p.ldb;
-  auto issue = [&](int buf) __attribute__((always_inline)) {
+  // The loads of a tile are issued in two halves, A right after the barrier that frees the buffer
+  // and B one chunk later: the LDS takes tile loads and fragment reads at the same time, and 64 KB
+  // arriving in one burst get in the way of the reads more than two bursts of 32 KB (measured 1 %).
+  auto issue_a = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < NIA; ++j)
       load_to_lds(a_base, offa[j], lds_base + 2u * (unsigned)(buf * A_ELEMS + (j * NW + wave) * RPI * STRIDE));
+    a_base += BK;
+  };
+  auto issue_b = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < NIB; ++j)
       load_to_lds(b_base, offb[j], lds_base + 2u * (unsigned)(STAGES * A_ELEMS + buf * B_ELEMS + (j * NW + wave) * RPI * STRIDE));
-    a_base += BK;
     b_base += BK;
+  };
+  auto issue = [&](int buf) __attribute__((always_inline)) {
+    issue_a(buf);
+    issue_b(buf);
   };
   // LDS byte addresses of this lane's fragments for each 16-wide K chunk of a step (block 0 of
   // the wavefront, ring buffer 0).  swz(row) is the same for all 32 x 32 blocks of a wavefront
@@ -573,7 +582,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
           __builtin_amdgcn_sched_barrier(0);
           __builtin_amdgcn_s_waitcnt(vmcnt_imm(0) & 0xc07f);  // vmcnt(0) and lgkmcnt(0)
           ring_barrier();
-          if (steady || t + 2 < nk) issue(cur);
+          if (steady || t + 2 < nk) issue_a(cur);
+        }
+        if (kk == CH - 1) {
+          if (steady || t + 2 < nk) issue_b(cur);
         }
       }
     };
@@ -612,7 +624,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
           if (steady || t + STAGES - 2 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 3) * INSTR));
           else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
           ring_barrier();
-          if (steady || t + STAGES - 1 < nk) issue(fill);
+          if (steady || t + STAGES - 1 < nk) issue_a(fill);
+        }
+        if (kk == CH - 1) {
+          if (steady || t + STAGES - 1 < nk) issue_b(fill);
         }
       }
     };
