@@ -278,6 +278,24 @@ int mi_loss_backward(mi_mlp* h);
 int mi_mlp_get_loss(mi_mlp* h, double* loss_per_replica, double* total);
 
 /*
+ * The loss front-end on caller-owned device buffers, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference; it is mi_loss_backward + mi_mlp_get_loss without a
+ * handle: the same kernel, same arithmetic and same summation order, hence the same bits.
+ *   dy[i]               = (pred[i] - label[i]) / batch_per_replica          (dtype of pred)
+ *   loss_per_replica[r] = (1/B) sum over replica r's rows of 0.5 * |pred_i - label_i|^2  (device, R doubles)
+ * pred, label and dy are dense [R*batch_per_replica x N]; pred and dy are fp32 (MI_F32) or bf16
+ * (MI_BF16), label is fp32.  The kernel's partial sums live in a device-resident static array of
+ * 512 KB (64 doubles per replica) that each GPU the library runs on holds until the process ends;
+ * the call performs no hipMalloc / hipFree and fails with MI_ERR_INVALID for R > 1024.  The address
+ * of the array is looked up on the first call on each device: make that call outside a graph
+ * capture.  All calls on one GPU share the array, so calls that overlap in time on one GPU (two
+ * streams, two threads) race; calls ordered on one stream do not.  Asynchronous on `stream`.
+ */
+int mi_l2_loss_static(int dtype, int R, int batch_per_replica, int N, const void* pred, const float* label,
+                      void* dy, double* loss_per_replica, void* stream);
+
+/*
  * Runs one step (like mi_mlp_step, eagerly, on the configured two-stream schedule) with an event
  * pair around every launch and writes the timeline to `path` in the format of the reference's
  * trace.log (mlp_tbb.cc:85-104,1379-1392: a JSON array of begin/end records with ts in

@@ -85,6 +85,7 @@ SIGNATURES = {
     "mi_loss_backward": [c_void_p],
     "mi_mlp_get_loss": [c_void_p, POINTER(c_double), POINTER(c_double)],
     "mi_mlp_trace_step": [c_void_p, c_float, c_char_p],
+    "mi_l2_loss_static": [c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
 }
 
 _lib = None

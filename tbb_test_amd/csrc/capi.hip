@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -394,6 +395,45 @@ int op_loss(mi_mlp* h, hipStream_t s) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e, "loss launch");
   return ts.finish();
+}
+
+// ---- loss front-end on caller-owned buffers, allocating nothing --------------------------------
+// The partial sums of l2_loss_kernel are the one scratch buffer of the loss path (the handle keeps
+// them in loss_partials, allocated by mi_mlp_set_labels).  mi_l2_loss_static keeps them in this
+// device-resident array instead, so that callers which cannot allocate can use the loss kernel.
+// In host code the array's name is only a stand-in: the address of each device's copy is asked
+// for once per device (static_scratch_of) and that pointer is what the kernels receive.
+constexpr int LOSS_STATIC_MAX_REPLICAS = 1024;
+static __device__ __align__(256) double g_loss_scratch[(size_t)LOSS_STATIC_MAX_REPLICAS * LOSS_CHUNKS];  // 512 KB per device
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+double* g_scratch_ptr[MAX_DEVICES] = {};  // per device: address of that device's g_loss_scratch
+
+int static_scratch_of_current_device(double** out) {
+  int dev = -1;
+  MI_HIP(hipGetDevice(&dev));
+  MI_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "device index %d beyond the %d this library tracks", dev, MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    MI_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_loss_scratch)));
+    MI_REQUIRE(p != nullptr, "hipGetSymbolAddress returned a null address for the loss scratch");
+    g_scratch_ptr[dev] = static_cast<double*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return MI_OK;
+}
+
+// loss[r] = (sum of replica r's partial sums, in chunk order) / B -- the fold mi_mlp_get_loss does
+// on the host, same order and same operations, so both give the same bits.
+__global__ __launch_bounds__(64) void loss_fold_kernel(const double* __restrict__ partials, double* __restrict__ loss,
+                                                       int R, double batch) {
+  const int r = blockIdx.x * 64 + threadIdx.x;
+  if (r >= R) return;
+  double acc = 0.0;
+  for (int c = 0; c < LOSS_CHUNKS; ++c) acc += partials[(size_t)r * LOSS_CHUNKS + c];
+  loss[r] = acc / batch;
 }
 
 // Enqueues one whole step.
@@ -933,6 +973,35 @@ int mi_mlp_get_loss(mi_mlp* h, double* loss_per_replica, double* total) {
     sum += acc;
   }
   if (total) *total = sum;
+  return MI_OK;
+}
+
+int mi_l2_loss_static(int dtype, int R, int batch_per_replica, int N, const void* pred, const float* label, void* dy,
+                      double* loss_per_replica, void* stream) {
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "dtype must be MI_F32 or MI_BF16 (got %d)", dtype);
+  MI_REQUIRE(R >= 1 && batch_per_replica >= 1 && N >= 1, "R, batch_per_replica and N must be positive (got %d, %d, %d)",
+             R, batch_per_replica, N);
+  MI_REQUIRE(R <= LOSS_STATIC_MAX_REPLICAS, "R = %d exceeds the %d replicas the static scratch holds", R,
+             LOSS_STATIC_MAX_REPLICAS);
+  MI_REQUIRE(pred && label && dy && loss_per_replica, "null pointer");
+  double* scratch = nullptr;
+  if (int rc = static_scratch_of_current_device(&scratch)) return rc;
+  hipStream_t s = as_stream(stream);
+  const size_t per_replica = (size_t)batch_per_replica * N;
+  const float inv_b = 1.0f / (float)batch_per_replica;
+  // every block of the grid stores its partial sum, so the scratch needs no clearing between calls
+  if (dtype == MI_F32)
+    mi::launch_kernel(l2_loss_kernel<false>, dim3(LOSS_CHUNKS, R), dim3(256), 0, s, dy, pred, label, per_replica, inv_b,
+                      scratch);
+  else
+    mi::launch_kernel(l2_loss_kernel<true>, dim3(LOSS_CHUNKS, R), dim3(256), 0, s, dy, pred, label, per_replica, inv_b,
+                      scratch);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e, "loss launch");
+  mi::launch_kernel(loss_fold_kernel, dim3((R + 63) / 64), dim3(64), 0, s, (const double*)scratch, loss_per_replica, R,
+                    (double)batch_per_replica);
+  e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e, "loss fold launch");
   return MI_OK;
 }
 
