@@ -14,7 +14,9 @@
  *     torch tensor's data_ptr()); "host pointer" = ordinary pageable or pinned host memory.
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Raw operations are
  *     asynchronous with respect to the host.
- *   - a handle is not thread-safe; distinct handles may be used from distinct threads.
+ *   - a handle is not thread-safe; distinct handles may be used from distinct threads (the
+ *     library's own process-wide state -- kernel attributes per device, the tuning hooks -- is
+ *     synchronised; mi_last_error() is per thread).
  */
 #ifndef MI_MLP_H
 #define MI_MLP_H
@@ -56,6 +58,12 @@ typedef enum mi_dtype {
                                     except for models whose GEMMs have four or more 128 x 128
                                     tiles per CU and fill the device on their own */
 
+#define MI_FLAG_KEEP_GRADIENTS 0x10u /* every layer's dZ (gradient w.r.t. the layer's pre-activation
+                                    output) keeps a buffer of its own, so that mi_mlp_get_dz answers
+                                    for every layer after a whole step; default: three buffers in
+                                    rotation.  Same kernels, same stream dependencies, same results;
+                                    costs (L-3) * R*B * max width elements of HBM.  For verification. */
+
 /* Timing slots, same names and order as the reference's enum Breakdown
  * (mlp_bench_common.h:12-20). */
 enum {
@@ -86,7 +94,8 @@ int mi_stream_sync(void* stream);
 
 /* Tuning hook: force tile configuration `variant` of the MFMA GEMM for kind 0 (nt), 1 (nn) or
  * 2 (tn); 0 restores the automatic choice.  A shape the forced configuration cannot tile falls
- * back to the any-shape kernel.  Process-wide; not meant for production callers. */
+ * back to the any-shape kernel.  Process-wide; a handle that already captured its step graph
+ * captures it again before the next replay.  Not meant for production callers. */
 int mi_set_gemm_variant(int kind, int variant);
 
 /* ------------------------------------------------------------------------------------------ */
@@ -196,7 +205,8 @@ typedef struct mi_mlp mi_mlp;
  * [nfeatures[l+1] x nfeatures[l]] as at mlp_omp.cc:395-396), R data-parallel replicas of
  * batch_per_replica rows each (replica r owns rows [r*B, (r+1)*B) of every activation, the
  * split of Partition.cc:25-27).  Device state: one parameter arena (all W_l and b_l), R gradient
- * arenas of the same layout, L+1 activation buffers and two gradient ping-pong buffers.
+ * arenas of the same layout, L+1 activation buffers and three rotating dZ buffers (bf16 models
+ * add the bf16 weight copies W, W^T and the transposed operand copies of the weight gradient).
  * Stands in for the allocation block of main(), mlp_omp.cc:390-409.
  */
 int mi_mlp_create(mi_mlp** h, int L, const int* nfeatures, int batch_per_replica, int R, int dtype,
@@ -233,8 +243,10 @@ int mi_mlp_get_wgrad(mi_mlp* h, int l, int r, float* dst, int ld);
 int mi_mlp_get_bgrad(mi_mlp* h, int l, int r, float* dst);
 int mi_mlp_get_dx(mi_mlp* h, float* dst, int ld);
 /* Gradient with respect to the pre-activation output of layer l, [R*B x N_{l+1}]: the uploaded dY
- * for l = L-1, otherwise what mi_fc_dgrad(l+1) produced.  The two gradient buffers alternate, so
- * the value is only meaningful between mi_fc_dgrad(l+1) and mi_fc_dgrad(l-1). */
+ * for l = L-1, otherwise what mi_fc_dgrad(l+1) produced.  dZ_l lives in buffer l mod 3 of a
+ * rotation of three, so the value is meaningful from mi_fc_dgrad(l+1) until mi_fc_dgrad(l-2)
+ * overwrites it (after a whole step: layers 0, 1, 2 and L-1); with MI_FLAG_KEEP_GRADIENTS every
+ * layer keeps its own buffer and the value stays until the next step. */
 int mi_mlp_get_dz(mi_mlp* h, int l, float* dst, int ld);
 
 /* Device-side copy of all weights and biases (snapshot) and its inverse (restore), both
@@ -243,6 +255,21 @@ int mi_mlp_get_dz(mi_mlp* h, int l, float* dst, int ld);
  * by benchmarking with alpha = 1e-10 (mlp_omp.cc:609,699,718). */
 int mi_mlp_snapshot_weights(mi_mlp* h);
 int mi_mlp_restore_weights(mi_mlp* h);
+
+/* bf16 models: the bf16 copy of W_l that the forward GEMM reads (transposed = 0, [N_{l+1} x N_l])
+ * or the transposed copy W_l^T that the input-gradient GEMM reads (transposed = 1,
+ * [N_l x N_{l+1}]), widened to fp32.  Both are rewritten by every update.  Synchronous. */
+int mi_mlp_get_weight_shadow(mi_mlp* h, int l, int transposed, float* dst, int ld);
+
+/* What the last mi_mlp_step / mi_mlp_trace_step actually did (the scheduling flags are requests;
+ * the library also looks at the shapes and at whether per-kernel timing is on):
+ *   info[0]  1 = backward pass on two streams, 0 = on one
+ *   info[1]  1 = one update launch per layer on the second stream, 0 = one launch at the end
+ *   info[2]  1 = steps replay a captured HIP graph
+ *   info[3]  bf16 models: how many of the 2(L-1) transposed operand copies of the weight-gradient
+ *            GEMMs were written by the epilogue of the GEMM that produced the operand (the rest
+ *            came from separate transpose launches); 0 for fp32 models */
+int mi_mlp_get_schedule(mi_mlp* h, int* info);
 
 /* Number of parameters P = sum_l (N_l*N_{l+1} + N_{l+1}) and the padded element stride between
  * consecutive replicas' gradient arenas. */

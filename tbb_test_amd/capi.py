@@ -12,7 +12,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
 MI_F32, MI_BF16 = 0, 1
-FLAG_RELU_LAST, FLAG_NO_GRAPH, FLAG_PER_LAYER_UPDATE, FLAG_SERIAL_BACKWARD = 1, 2, 4, 8
+FLAG_RELU_LAST, FLAG_NO_GRAPH, FLAG_PER_LAYER_UPDATE, FLAG_SERIAL_BACKWARD, FLAG_KEEP_GRADIENTS = 1, 2, 4, 8, 16
 BREAKDOWN_NAMES = ("fwd", "wgt_grad", "bwd", "wgt_update", "wgt_update_reduce_scatter", "wgt_update_allgather")
 NUM_BREAKDOWNS = len(BREAKDOWN_NAMES)
 
@@ -78,6 +78,8 @@ SIGNATURES = {
     "mi_mlp_snapshot_weights": [c_void_p],
     "mi_mlp_restore_weights": [c_void_p],
     "mi_mlp_param_count": [c_void_p, POINTER(c_size_t), POINTER(c_size_t)],
+    "mi_mlp_get_weight_shadow": [c_void_p, c_int, c_int, c_void_p, c_int],
+    "mi_mlp_get_schedule": [c_void_p, POINTER(c_int)],
     "mi_mlp_enable_timing": [c_void_p, c_int],
     "mi_mlp_reset_timings": [c_void_p],
     "mi_mlp_get_timings": [c_void_p, POINTER(c_double), POINTER(c_longlong)],
@@ -254,6 +256,18 @@ class MlpHandle:
     def bgrad_of(self, l, r): return self._get(lib().mi_mlp_get_bgrad, (self.nf[l + 1],), l, r)
     def dx(self): return self._get(lib().mi_mlp_get_dx, (self.MB, self.nf[0]))
     def dz(self, l): return self._get(lib().mi_mlp_get_dz, (self.MB, self.nf[l + 1]), l)
+
+    def weight_shadow(self, l, transposed=False):
+        """bf16 models: the bf16 copy of W_l (or of W_l^T) the GEMMs read, widened to fp32."""
+        shape = (self.nf[l], self.nf[l + 1]) if transposed else (self.nf[l + 1], self.nf[l])
+        return self._get(lib().mi_mlp_get_weight_shadow, shape, l, int(transposed))
+
+    def schedule(self):
+        """What the last step did: dict(dual_streams, per_layer_update, graph, fused_transposes)."""
+        info = (c_int * 4)()
+        check(lib().mi_mlp_get_schedule(self._h, info))
+        return {"dual_streams": bool(info[0]), "per_layer_update": bool(info[1]), "graph": bool(info[2]),
+                "fused_transposes": int(info[3])}
 
     def snapshot_weights(self): check(lib().mi_mlp_snapshot_weights(self._h))
     def restore_weights(self): check(lib().mi_mlp_restore_weights(self._h))

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -44,8 +45,12 @@ int hip_fail(hipError_t e, const char* what) {
     if (!(cond)) return fail(MI_ERR_INVALID, __VA_ARGS__); \
   } while (0)
 
-int g_variant[3] = {0, 0, 0};  // forced tile configuration per GEMM kind (nt, nn, tn); 0 = automatic
-int g_hvariant = 0;             // forced tile configuration of the bf16 kernel
+// Tuning hooks, process-wide: forced tile configuration per fp32 GEMM kind (nt, nn, tn) and of the
+// bf16 kernel; 0 = automatic.  A change bumps the epoch, and a handle whose captured graph is older
+// re-captures before its next replay.
+std::atomic<int> g_variant[3] = {{0}, {0}, {0}};
+std::atomic<int> g_hvariant{0};
+std::atomic<int> g_variant_epoch{0};
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
@@ -72,14 +77,17 @@ struct mi_mlp {
   uint16_t* params16_saved = nullptr;
   uint16_t* params16T_saved = nullptr;
   std::vector<uint16_t*> actsT;  // bf16 only: per-replica transposed activations [R][N_l x B], l < L
-  // bf16 only: per-replica transposed gradients [R][max N x B]; dZ_l^T lives in dzT[l % 3] like
-  // dZ_l in dz[l % 3].  *_fused: the producing GEMM wrote the transposed copy in its epilogue.
-  uint16_t* dzT[3] = {nullptr, nullptr, nullptr};
+  // Gradient buffers: dZ_l lives in dz[l % ndz]; ndz = 3 (a rotation: dZ_l is dead once wgrad(l) and
+  // dgrad(l) have read it) or, with MI_FLAG_KEEP_GRADIENTS, one buffer per layer.
+  int ndz = 3;
+  // bf16 only: per-replica transposed gradients [R][max N x B]; dZ_l^T lives in dzT[l % ndz] like
+  // dZ_l in dz[l % ndz].  *_fused: the producing GEMM wrote the transposed copy in its epilogue.
+  std::vector<uint16_t*> dzT;
   std::vector<char> actsT_fused;  // [L]
-  bool dzT_fused[3] = {false, false, false};
+  std::vector<char> dzT_fused;  // [ndz]
   std::vector<void*> acts;    // L+1 buffers [MB x nf[l]], fp32 or bf16
   void* dy = nullptr;         // upstream gradient [MB x nf[L]]
-  void* dz[3] = {nullptr, nullptr, nullptr};  // gradient rotation [MB x max width]: dZ_l lives in dz[l % 3]
+  std::vector<void*> dz;      // [ndz] buffers of [MB x max width]
   void* dx = nullptr;         // gradient w.r.t. the input [MB x nf[0]]
   float* staging = nullptr;   // fp32 bounce buffer for bf16 uploads/downloads [MB x max width] or one W
   size_t staging_elems = 0;
@@ -110,8 +118,15 @@ struct mi_mlp {
 
   // graph replay
   hipGraphExec_t graph_exec = nullptr;
-  float graph_lr = 0.0f;
+  int graph_epoch = 0;  // g_variant_epoch at capture time
   int eager_steps = 0;
+  // -lr on the device: the update kernels of a step read it from here, so that a captured graph
+  // follows a learning-rate schedule without being captured again
+  float* neg_lr_dev = nullptr;
+  float neg_lr_value = 0.0f;
+  bool neg_lr_valid = false;
+  // what the last enqueue_step decided (mi_mlp_get_schedule)
+  bool last_dual = false, last_per_layer = false;
 
   size_t esize() const { return dtype == MI_BF16 ? 2 : 4; }
   size_t maxw() const {
@@ -199,7 +214,7 @@ struct TimedScope {
 const void* dz_of_layer(mi_mlp* h, int l) {
   // gradient w.r.t. the pre-activation output of layer l
   if (l == h->L - 1 && !(h->flags & MI_FLAG_RELU_LAST)) return h->dy;
-  return h->dz[l % 3];
+  return h->dz[l % h->ndz];
 }
 
 int op_forward(mi_mlp* h, int l, hipStream_t s) {
@@ -238,12 +253,12 @@ int op_wgrad(mi_mlp* h, int l, hipStream_t s, bool with_bias) {
     const int B = h->B, nin = h->nf[l], nout = h->nf[l + 1];
     // (each copy comes from the epilogue of the GEMM that produced the operand when that was
     // possible, else from a transpose here)
-    uint16_t* dzt = h->dzT[l % 3];
+    uint16_t* dzt = h->dzT[l % h->ndz];
     e = hipSuccess;
     if (!h->actsT_fused[l])
       e = mi::transpose_bf16(h->R, B, nin, (const uint16_t*)h->acts[l], nin, (long long)B * nin, h->actsT[l], B,
                              (long long)nin * B, s);
-    const bool dz_fused = l < h->L - 1 && h->dzT_fused[l % 3];  // the last layer's dZ is the given or derived dY
+    const bool dz_fused = l < h->L - 1 && h->dzT_fused[l % h->ndz];  // the last layer's dZ is the given or derived dY
     if (e == hipSuccess && !dz_fused)
       e = mi::transpose_bf16(h->R, B, nout, (const uint16_t*)dz_of_layer(h, l), nout, (long long)B * nout, dzt, B,
                              (long long)nout * B, s);
@@ -261,9 +276,9 @@ int op_bgrad(mi_mlp* h, int l, hipStream_t s) {
   if (h->dtype != MI_F32) {
     const int B = h->B, nout = h->nf[l + 1];
     hipError_t eb = mi::transpose_bf16(h->R, B, nout, (const uint16_t*)dz_of_layer(h, l), nout, (long long)B * nout,
-                                       h->dzT[l % 3], B, (long long)nout * B, s);
+                                       h->dzT[l % h->ndz], B, (long long)nout * B, s);
     if (eb == hipSuccess)
-      eb = mi::rowsum_bf16(h->R, nout, B, h->dzT[l % 3], B, (long long)nout * B, h->grads + h->boff[l],
+      eb = mi::rowsum_bf16(h->R, nout, B, h->dzT[l % h->ndz], B, (long long)nout * B, h->grads + h->boff[l],
                            (long long)h->stride, s);
     if (eb != hipSuccess) return hip_fail(eb, "bias-gradient launch");
     return MI_OK;
@@ -277,20 +292,20 @@ int op_bgrad(mi_mlp* h, int l, hipStream_t s) {
 int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
   TimedScope ts(h, s, MI_BWD, l);
   if (ts.status) return ts.status;
-  void* out = (l == 0) ? h->dx : h->dz[(l - 1) % 3];
+  void* out = (l == 0) ? h->dx : h->dz[(l - 1) % h->ndz];
   const void* mask = (l == 0) ? nullptr : h->acts[l];
   hipError_t e;
   if (h->dtype == MI_F32) {
     e = mi::sgemm_nn(h->MB, h->nf[l], h->nf[l + 1], (const float*)dz_of_layer(h, l), h->nf[l + 1],
                      h->params + h->woff[l], h->nf[l], (float*)out, h->nf[l], (const float*)mask, h->nf[l], s,
-                     g_variant[1] ? g_variant[1] : (h->corun ? 100 : 0));
+                     g_variant[1].load() ? g_variant[1].load() : (h->corun ? 100 : 0));
   } else {
     bool wrote = false;
-    uint16_t* ct = (l > 0) ? h->dzT[(l - 1) % 3] : nullptr;  // dZ_{l-1}^T for the weight gradient of layer l-1
+    uint16_t* ct = (l > 0) ? h->dzT[(l - 1) % h->ndz] : nullptr;  // dZ_{l-1}^T for the weight gradient of layer l-1
     e = mi::hgemm_nt(1, h->MB, h->nf[l], h->nf[l + 1], (const uint16_t*)dz_of_layer(h, l), h->nf[l + 1], 0,
                      h->params16T + h->woff[l], h->nf[l + 1], 0, out, h->nf[l], 0, mask ? 2 : 3, nullptr, 0,
                      (const uint16_t*)mask, h->nf[l], s, g_hvariant, ct, h->B, &wrote);
-    if (l > 0) h->dzT_fused[(l - 1) % 3] = wrote;
+    if (l > 0) h->dzT_fused[(l - 1) % h->ndz] = wrote;
   }
   if (e != hipSuccess) return hip_fail(e, "input-gradient GEMM launch");
   return ts.finish();
@@ -307,7 +322,7 @@ int op_update(mi_mlp* h, int l_or_all, float lr, hipStream_t s) {
   TimedScope ts(h, s, MI_WGT_UPDATE, l_or_all >= 0 ? layer_slot : -1);
   if (ts.status) return ts.status;
   hipError_t e = mi::reduce_sgd(h->params + off, h->params16 ? h->params16 + off : nullptr, h->grads + off, n,
-                                h->stride, h->R, lr, s);
+                                h->stride, h->R, lr, s, h->neg_lr_dev);
   if (e != hipSuccess) return hip_fail(e, "reduce+SGD launch");
   if (h->params16T) {  // refresh the transposed bf16 weight copies the input-gradient GEMMs read
     const int first = l_or_all >= 0 ? l_or_all : 0, last = l_or_all >= 0 ? l_or_all : h->L - 1;
@@ -333,7 +348,7 @@ int op_last_mask(mi_mlp* h, hipStream_t s) {
   const size_t n = (size_t)h->MB * h->nf[h->L];
   size_t blocks = (n + 255) / 256;
   if (blocks > 4096) blocks = 4096;
-  mi::launch_kernel(mask_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float*)h->dz[(h->L - 1) % 3],
+  mi::launch_kernel(mask_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float*)h->dz[(h->L - 1) % h->ndz],
                      (const float*)h->dy, (const float*)h->acts[h->L], n);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e, "mask launch");
@@ -395,6 +410,21 @@ int op_loss(mi_mlp* h, hipStream_t s) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e, "loss launch");
   return ts.finish();
+}
+
+__global__ void set_scalar_kernel(float* dst, float v) { *dst = v; }
+
+// Makes *neg_lr_dev = -lr for the update launches that follow on the handle's streams.  Called
+// outside any capture (the value is not part of the graph) and only when lr changes.  Ordered:
+// it runs on the main stream, which every step joins the second stream into at its end.
+int ensure_lr(mi_mlp* h, float lr) {
+  if (h->neg_lr_valid && h->neg_lr_value == -lr) return MI_OK;
+  hipLaunchKernelGGL(set_scalar_kernel, dim3(1), dim3(1), 0, h->stream, h->neg_lr_dev, -lr);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e, "learning-rate launch");
+  h->neg_lr_value = -lr;
+  h->neg_lr_valid = true;
+  return MI_OK;
 }
 
 // ---- loss front-end on caller-owned buffers, allocating nothing --------------------------------
@@ -465,6 +495,8 @@ int enqueue_step(mi_mlp* h, float lr) {
   // 3, 1024 tiles: 11.32 ms with one backward stream, 11.47 ms with two; config 5: 45.9 / 47.1 ms).
   const bool crowded = (long long)(h->MB / 128) * (long long)(h->maxw() / 128) >= 1024;
   const bool dual = !(h->flags & MI_FLAG_SERIAL_BACKWARD) && !h->timing && !crowded;
+  h->last_dual = dual;
+  h->last_per_layer = per_layer;
   hipStream_t s2 = dual ? h->stream2 : s;
   if (dual) {  // fork: dZ_{L-1} and all activations are ready
     MI_HIP(hipEventRecord(h->ev_fork, s));
@@ -602,7 +634,8 @@ int mi_stream_sync(void* stream) {
 
 int mi_set_gemm_variant(int kind, int variant) {
   MI_REQUIRE(kind >= 0 && kind < 3, "kind must be 0 (nt), 1 (nn) or 2 (tn)");
-  g_variant[kind] = variant;
+  g_variant[kind].store(variant);
+  g_variant_epoch.fetch_add(1);
   return MI_OK;
 }
 
@@ -737,7 +770,8 @@ int mi_rowsum_bf16(int batch, int rows, int cols, const void* src, int ld, long 
 }
 
 int mi_set_hgemm_variant(int variant) {
-  g_hvariant = variant;
+  g_hvariant.store(variant);
+  g_variant_epoch.fetch_add(1);
   return MI_OK;
 }
 
@@ -790,6 +824,7 @@ int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_repli
   h->dtype = dtype;
   h->flags = flags;
   h->nf.assign(nfeatures, nfeatures + L + 1);
+  h->ndz = (flags & MI_FLAG_KEEP_GRADIENTS) ? std::max(L, 3) : 3;
   h->woff.resize(L);
   h->boff.resize(L);
   size_t off = 0;
@@ -814,13 +849,16 @@ int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_repli
   };
   const size_t es = h->esize();
   alloc((void**)&h->params, h->stride * 4);
+  alloc((void**)&h->neg_lr_dev, 256);
   alloc((void**)&h->grads, h->stride * 4 * (size_t)R);
   if (dtype == MI_BF16) {
     alloc((void**)&h->params16, h->stride * 2);
     alloc((void**)&h->params16T, h->stride * 2);
     h->actsT.assign(L, nullptr);
     for (int l = 0; l < L; ++l) alloc((void**)&h->actsT[l], (size_t)h->MB * h->nf[l] * 2);
-    for (int i = 0; i < 3; ++i) alloc((void**)&h->dzT[i], (size_t)h->MB * h->maxw() * 2);
+    h->dzT.assign(h->ndz, nullptr);
+    h->dzT_fused.assign(h->ndz, 0);
+    for (int i = 0; i < h->ndz; ++i) alloc((void**)&h->dzT[i], (size_t)h->MB * h->maxw() * 2);
     h->actsT_fused.assign(L, 0);
     size_t wmax = 0;
     for (int l = 0; l < L; ++l) wmax = std::max(wmax, (size_t)h->nf[l] * h->nf[l + 1]);
@@ -830,7 +868,8 @@ int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_repli
   h->acts.assign(L + 1, nullptr);
   for (int l = 0; l <= L; ++l) alloc(&h->acts[l], (size_t)h->MB * h->nf[l] * es);
   alloc(&h->dy, (size_t)h->MB * h->nf[L] * es);
-  for (int i = 0; i < 3; ++i) alloc(&h->dz[i], (size_t)h->MB * h->maxw() * es);
+  h->dz.assign(h->ndz, nullptr);
+  for (int i = 0; i < h->ndz; ++i) alloc(&h->dz[i], (size_t)h->MB * h->maxw() * es);
   alloc(&h->dx, (size_t)h->MB * h->nf[0] * es);
   if (rc == MI_OK && hipDeviceSynchronize() != hipSuccess) rc = fail(MI_ERR_HIP, "hipDeviceSynchronize failed");
   if (rc == MI_OK && hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking) != hipSuccess)
@@ -874,6 +913,7 @@ int mi_mlp_destroy(mi_mlp* h) {
   if (h->ev_join) (void)hipEventDestroy(h->ev_join);
   if (h->ev_fork) (void)hipEventDestroy(h->ev_fork);
   (void)hipFree(h->params);
+  (void)hipFree(h->neg_lr_dev);
   (void)hipFree(h->grads);
   (void)hipFree(h->params16);
   (void)hipFree(h->params_saved);
@@ -881,10 +921,10 @@ int mi_mlp_destroy(mi_mlp* h) {
   (void)hipFree(h->params16T);
   (void)hipFree(h->params16T_saved);
   for (auto a : h->actsT) (void)hipFree(a);
-  for (int i = 0; i < 3; ++i) (void)hipFree(h->dzT[i]);
+  for (auto a : h->dzT) (void)hipFree(a);
   for (void* a : h->acts) (void)hipFree(a);
   (void)hipFree(h->dy);
-  for (int i = 0; i < 3; ++i) (void)hipFree(h->dz[i]);
+  for (void* a : h->dz) (void)hipFree(a);
   (void)hipFree(h->dx);
   (void)hipFree(h->staging);
   (void)hipFree(h->labels);
@@ -903,7 +943,10 @@ int mi_mlp_set_weights(mi_mlp* h, int l, const float* W, int ld, const float* b)
   if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
   if (int rc = upload_matrix(h, h->params + h->woff[l], W, h->nf[l + 1], h->nf[l], ld, false)) return rc;
   if (b) {
-    MI_HIP(hipMemcpy(h->params + h->boff[l], b, (size_t)h->nf[l + 1] * 4, hipMemcpyHostToDevice));
+    // on the handle's stream (the streams are non-blocking: a null-stream copy would not be
+    // ordered against work still in flight on them)
+    MI_HIP(hipMemcpyAsync(h->params + h->boff[l], b, (size_t)h->nf[l + 1] * 4, hipMemcpyHostToDevice, h->stream));
+    MI_HIP(hipStreamSynchronize(h->stream));
   } else {
     MI_HIP(hipMemsetAsync(h->params + h->boff[l], 0, (size_t)h->nf[l + 1] * 4, h->stream));
     MI_HIP(hipStreamSynchronize(h->stream));
@@ -1017,6 +1060,7 @@ int mi_mlp_trace_step(mi_mlp* h, float lr, const char* path) {
   h->trace_items.clear();
   int rc = MI_OK;
   if (hipEventRecord(base, h->stream) != hipSuccess) rc = fail(MI_ERR_HIP, "hipEventRecord failed");
+  if (rc == MI_OK) rc = ensure_lr(h, lr);
   if (rc == MI_OK) rc = enqueue_step(h, lr);
   h->tracing = false;
   h->eager_steps++;
@@ -1082,10 +1126,12 @@ int mi_fc_dgrad(mi_mlp* h, int l) {
 }
 int mi_reduce_sgd(mi_mlp* h, float lr) {
   if (int rc = check_handle(h)) return rc;
+  if (int rc = ensure_lr(h, lr)) return rc;
   return op_update(h, -1, lr, h->stream);
 }
 int mi_reduce_sgd_layer(mi_mlp* h, int l, float lr) {
   if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  if (int rc = ensure_lr(h, lr)) return rc;
   return op_update(h, l, lr, h->stream);
 }
 
@@ -1096,10 +1142,13 @@ int mi_mlp_step(mi_mlp* h, float lr) {
     // the first step always runs eagerly: it performs the one-time kernel attribute setup,
     // which must not happen inside a stream capture
     h->eager_steps++;
+    if (int rc = ensure_lr(h, lr)) return rc;
     return enqueue_step(h, lr);
   }
-  if (h->graph_exec && h->graph_lr != lr) drop_graph(h);
+  if (int rc = ensure_lr(h, lr)) return rc;
+  if (h->graph_exec && h->graph_epoch != g_variant_epoch.load()) drop_graph(h);
   if (!h->graph_exec) {
+    const int epoch = g_variant_epoch.load();
     hipGraph_t graph = nullptr;
     MI_HIP(hipStreamBeginCapture(h->stream, hipStreamCaptureModeThreadLocal));
     int rc = enqueue_step(h, lr);
@@ -1115,7 +1164,7 @@ int mi_mlp_step(mi_mlp* h, float lr) {
       h->graph_exec = nullptr;
       return hip_fail(e, "hipGraphInstantiate");
     }
-    h->graph_lr = lr;
+    h->graph_epoch = epoch;
   }
   MI_HIP(hipGraphLaunch(h->graph_exec, h->stream));
   return MI_OK;
@@ -1182,6 +1231,29 @@ int mi_mlp_restore_weights(mi_mlp* h) {
 int mi_mlp_get_dz(mi_mlp* h, int l, float* dst, int ld) {
   if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
   return download_matrix(h, dst, dz_of_layer(h, l), h->MB, h->nf[l + 1], ld, h->dtype == MI_BF16);
+}
+
+int mi_mlp_get_schedule(mi_mlp* h, int* info) {
+  if (int rc = check_handle(h)) return rc;
+  MI_REQUIRE(info != nullptr, "null output pointer");
+  MI_REQUIRE(h->eager_steps > 0, "no step has run yet");
+  info[0] = h->last_dual ? 1 : 0;
+  info[1] = h->last_per_layer ? 1 : 0;
+  info[2] = h->graph_exec ? 1 : 0;
+  int fused = 0;
+  if (h->dtype == MI_BF16) {
+    for (int l = 1; l < h->L; ++l) fused += h->actsT_fused[l] ? 1 : 0;  // A_l^T written by forward(l-1)
+    for (int l = 0; l + 1 < h->L; ++l) fused += h->dzT_fused[l % h->ndz] ? 1 : 0;  // dZ_l^T written by dgrad(l+1)
+  }
+  info[3] = fused;
+  return MI_OK;
+}
+
+int mi_mlp_get_weight_shadow(mi_mlp* h, int l, int transposed, float* dst, int ld) {
+  if (int rc = check_layer(h, l, h ? h->L - 1 : 0)) return rc;
+  MI_REQUIRE(h->dtype == MI_BF16, "only bf16 models keep bf16 weight copies");
+  if (transposed) return download_matrix(h, dst, h->params16T + h->woff[l], h->nf[l], h->nf[l + 1], ld, true);
+  return download_matrix(h, dst, h->params16 + h->woff[l], h->nf[l + 1], h->nf[l], ld, true);
 }
 
 int mi_mlp_param_count(mi_mlp* h, size_t* params, size_t* replica_stride) {

@@ -704,13 +704,8 @@ static hipError_t launch_h(HGemmArgs& p, int batch, hipStream_t s) {
   constexpr size_t lds_bytes = STAGES * (size_t)(BM + BN) * BK * sizeof(u16);
   static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB of LDS");
   auto kern = gemm_bf16_mfma<BM, BN, BK, WM, WN, EPI, PF, STAGES>;
-  static bool attr_set = false;
-  if (lds_bytes > 64 * 1024 && !attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) return e;
   p.tiles_m = p.M / BM;
   p.tiles_n = p.N / BN;
   launch_kernel(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
@@ -722,13 +717,8 @@ static hipError_t launch_dma(HGemmArgs& p, int batch, hipStream_t s) {
   constexpr size_t lds_bytes = STAGES * (size_t)(BM + BN) * BK * sizeof(u16);
   static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB of LDS");
   auto kern = gemm_bf16_dma<BM, BN, BK, WM, WN, EPI, STAGES>;
-  static bool attr_set = false;
-  if (lds_bytes > 64 * 1024 && !attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) return e;
   p.tiles_m = p.M / BM;
   p.tiles_n = p.N / BN;
   launch_kernel(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);

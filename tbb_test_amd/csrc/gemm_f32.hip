@@ -985,13 +985,8 @@ static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
   using TB = TileShape<BN, BK, BKM>;
   constexpr size_t lds_bytes = STAGES * (TA::kFloats + TB::kFloats) * sizeof(float);
   auto kern = gemm_f32_mfma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES, PF, GUARD>;
-  static bool attr_set = false;  // opt in to more than 64 KiB of dynamic LDS once per kernel
-  if (lds_bytes > 64 * 1024 && !attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) return e;
   p.tiles_m = GUARD ? (p.M + BM - 1) / BM : p.M / BM;
   p.tiles_n = GUARD ? (p.N + BN - 1) / BN : p.N / BN;
   set_raster(p, batch);
@@ -1011,13 +1006,8 @@ static hipError_t launch_dma(GemmArgs& p, int batch, hipStream_t s, bool exclusi
   constexpr size_t kExclusiveBytes = 84 * 1024;
   const size_t request = exclusive && lds_bytes < kExclusiveBytes ? kExclusiveBytes : lds_bytes;
   auto kern = gemm_f32_dma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES>;
-  static size_t attr_bytes = 0;  // opt in to more than 64 KiB of dynamic LDS, per kernel
-  if (request > 64 * 1024 && request > attr_bytes) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)request);
-    if (e != hipSuccess) return e;
-    attr_bytes = request;
-  }
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), request); e != hipSuccess) return e;
   p.tiles_m = p.M / BM;
   p.tiles_n = p.N / BN;
   set_raster(p, batch);

@@ -5,8 +5,10 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 
+#include <atomic>
 #include <cstddef>
 #include <cstdint>
+#include <mutex>
 
 namespace mi {
 
@@ -36,6 +38,34 @@ inline void launch_kernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_
   }
 }
 
+// Opt-in to more than 64 KiB of dynamic LDS for one kernel, remembered per device (the attribute
+// belongs to the kernel's code object on a device) and safe to reach from several host threads.
+// One object per kernel (a function-local static of the launcher template).  The attribute call
+// is made at most once per device and size, and never during a stream capture as long as the first
+// launch of each kernel happens outside one.
+struct LdsOptIn {
+  static constexpr int kMaxDevices = 64;
+  std::atomic<size_t> granted[kMaxDevices];
+  std::mutex mutex;
+  LdsOptIn() {
+    for (auto& g : granted) g.store(0, std::memory_order_relaxed);
+  }
+  hipError_t ensure(const void* kernel, size_t bytes) {
+    if (bytes <= 64 * 1024) return hipSuccess;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    if (granted[dev].load(std::memory_order_acquire) >= bytes) return hipSuccess;
+    std::lock_guard<std::mutex> lock(mutex);
+    if (granted[dev].load(std::memory_order_relaxed) >= bytes) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return e;
+    granted[dev].store(bytes, std::memory_order_release);
+    return hipSuccess;
+  }
+};
+
 // `variant` selects a tile configuration of the MFMA kernel (0 = choose from the shape, 100 =
 // choose from the shape knowing that another GEMM runs concurrently on a second stream); it is
 // exposed through mi_set_gemm_variant for tuning runs.
@@ -52,9 +82,11 @@ hipError_t sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const f
 hipError_t colsum_f32(int R, int M, int K, const float* A, int lda, float* out, long long stride_out,
                       hipStream_t s);
 
-// W[i] = fma(-lr, sum_r G[r*stride + i], W[i]); W16 (bf16 copy of the result) may be null
+// W[i] = fma(-lr, sum_r G[r*stride + i], W[i]); W16 (bf16 copy of the result) may be null.
+// neg_lr_dev (may be null): device address of -lr; when given, the kernel reads the factor from
+// there instead of taking `lr` -- a captured graph then follows a changing learning rate.
 hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t stride, int R, float lr,
-                      hipStream_t s);
+                      hipStream_t s, const float* neg_lr_dev = nullptr);
 
 // bf16: C = A[M,K] * B[N,K]^T with fp32 accumulation, both operands K-contiguous, blockIdx.z
 // batches with element strides batchA/B/C.  out_kind: 0 fp32 plain, 1 bf16 with bias + optional

@@ -34,8 +34,10 @@ __device__ __forceinline__ unsigned short f32_to_bf16_rne(float f) {
 template <int R_FIXED, bool WRITE_BF16, int UNROLL, bool STREAM>
 __global__ __launch_bounds__(256) void reduce_sgd_vec4(float* __restrict__ W, unsigned short* __restrict__ W16,
                                                        const float* __restrict__ G, size_t nvec,
-                                                       size_t stride_vec, int R_dyn, float neg_lr) {
+                                                       size_t stride_vec, int R_dyn, float neg_lr_arg,
+                                                       const float* __restrict__ neg_lr_dev) {
   const int R = R_FIXED > 0 ? R_FIXED : R_dyn;
+  const float neg_lr = neg_lr_dev ? *neg_lr_dev : neg_lr_arg;  // uniform: one scalar load
   const f32x4* __restrict__ g4 = reinterpret_cast<const f32x4*>(G);
   f32x4* __restrict__ w4 = reinterpret_cast<f32x4*>(W);
   auto ld = [&](const f32x4* ptr) { return STREAM ? __builtin_nontemporal_load(ptr) : *ptr; };
@@ -87,7 +89,9 @@ __global__ __launch_bounds__(256) void reduce_sgd_vec4(float* __restrict__ W, un
 // scalar version for unaligned arenas and for the tail that does not fill a float4
 __global__ __launch_bounds__(256) void reduce_sgd_scalar(float* __restrict__ W, unsigned short* __restrict__ W16,
                                                          const float* __restrict__ G, size_t begin, size_t n,
-                                                         size_t stride, int R, float neg_lr) {
+                                                         size_t stride, int R, float neg_lr_arg,
+                                                         const float* __restrict__ neg_lr_dev) {
+  const float neg_lr = neg_lr_dev ? *neg_lr_dev : neg_lr_arg;
   const size_t step = (size_t)gridDim.x * blockDim.x;
   for (size_t i = begin + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step) {
     float s = G[i];
@@ -106,7 +110,7 @@ static int grid_for(size_t work_items, int per_block, int max_blocks) {
 }
 
 hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t stride, int R, float lr,
-                      hipStream_t s) {
+                      hipStream_t s, const float* neg_lr_dev) {
   if (n == 0 || R <= 0) return hipSuccess;
   const float neg_lr = -lr;
   const bool vec = ((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(G)) & 15) == 0 &&
@@ -124,10 +128,10 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
   do {                                                                                                     \
     if (stream)                                                                                            \
       launch_kernel((reduce_sgd_vec4<RF, BF, 1, true>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, \
-                         stride / 4, R, neg_lr);                                                           \
+                         stride / 4, R, neg_lr, neg_lr_dev);                                               \
     else                                                                                                   \
       launch_kernel((reduce_sgd_vec4<RF, BF, 2, false>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, \
-                         stride / 4, R, neg_lr);                                                           \
+                         stride / 4, R, neg_lr, neg_lr_dev);                                               \
   } while (0)
 #define MI_LAUNCH_REDUCE(RF, BF) MI_LAUNCH_REDUCE2(RF, BF)
     if (W16) {
@@ -155,7 +159,7 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
   }
   if (done < n) {
     const int blocks = grid_for(n - done, 256, 2048);
-    launch_kernel(reduce_sgd_scalar, dim3(blocks), dim3(256), 0, s, W, W16, G, done, n, stride, R, neg_lr);
+    launch_kernel(reduce_sgd_scalar, dim3(blocks), dim3(256), 0, s, W, W16, G, done, n, stride, R, neg_lr, neg_lr_dev);
   }
   return hipGetLastError();
 }

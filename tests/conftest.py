@@ -24,6 +24,23 @@ def rel_err(actual, expected):
     return float(np.abs(actual - expected).max() / denom)
 
 
+def elem_err(actual, expected):
+    """Element-wise error max_i |a_i - e_i| / (|e_i| + rms(e)): unlike the norm-wise rel_err it sees a
+    wrong small entry next to large ones; the rms term keeps entries that cancel to (almost) zero
+    from demanding more than the accumulation can give."""
+    actual = np.asarray(actual, dtype=np.float64)
+    expected = np.asarray(expected, dtype=np.float64)
+    rms = float(np.sqrt(np.mean(expected * expected))) if expected.size else 0.0
+    if rms == 0.0:
+        return float(np.abs(actual).max()) if actual.size else 0.0
+    return float((np.abs(actual - expected) / (np.abs(expected) + rms)).max())
+
+
+def close(actual, expected, tol):
+    """Both bounds: norm-wise (the benchmark's stated tolerance) and element-wise."""
+    return rel_err(actual, expected) <= tol and elem_err(actual, expected) <= tol
+
+
 @pytest.fixture(scope="session")
 def mi():
     """The ctypes binding of libmi_mlp.so; fails (not skips) when the library is not built."""

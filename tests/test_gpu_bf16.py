@@ -145,7 +145,7 @@ STEP_CONFIGS = {
 }
 
 
-def _check_bf16_step(nf, B, R, flags, seed=31):
+def _check_bf16_step(nf, B, R, flags, seed=31, expect_fused=None):
     L = len(nf) - 1
     X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed=seed)
     rng = np.random.default_rng(1)
@@ -159,6 +159,8 @@ def _check_bf16_step(nf, B, R, flags, seed=31):
         h.snapshot_weights() if _ == 0 else h.restore_weights()
         h.step(LR)
     h.sync()
+    if expect_fused is not None:  # the transposed operand copies came out of the GEMM epilogues, not a fallback
+        assert h.schedule()["fused_transposes"] == expect_fused
     ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR)
     acts = [h.activation(l) for l in range(L + 1)]
     for l in range(L + 1):
@@ -188,15 +190,28 @@ def test_bf16_step_matches_fp32_oracle(name, flags):
     _check_bf16_step(nf, B, R, flags)
 
 
-@pytest.mark.parametrize("variant", [13, 19])
+@pytest.mark.parametrize("variant", [13, 17, 19])
 @pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, 0])
 def test_bf16_step_on_the_large_tile_kernels(variant, flags):
-    """The 256 x 256 direct-load kernels, which small models never pick by themselves: whole steps
-    with their fused transposed outputs and the ReLU mask tile brought into the LDS."""
+    """The direct-load kernels (256 x 256 and 128 x 128 tiles), which small models never pick by
+    themselves: whole steps against the full oracle with their fused transposed outputs (staged
+    through the LDS) and the ReLU mask tile brought into the LDS.  The per-replica batch is a
+    multiple of the tile height, which the fused transposed output needs; the test asserts that
+    all 2 (L-1) transposed copies were written by the GEMM epilogues."""
     lib = capi.lib()
     capi.check(lib.mi_set_hgemm_variant(variant))
     try:
-        _check_bf16_step([256, 512, 256, 512, 256], 128, 2, flags, seed=77)
+        nf = [256, 512, 256, 512, 256]
+        _check_bf16_step(nf, 256, 2, flags, seed=77, expect_fused=2 * (len(nf) - 2))
+    finally:
+        lib.mi_set_hgemm_variant(0)
+
+
+def test_bf16_step_falls_back_to_transpose_launches_when_the_batch_does_not_fit_the_tile():
+    lib = capi.lib()
+    capi.check(lib.mi_set_hgemm_variant(19))
+    try:
+        _check_bf16_step([256, 512, 256], 128, 2, capi.FLAG_NO_GRAPH, seed=78, expect_fused=0)
     finally:
         lib.mi_set_hgemm_variant(0)
 
