@@ -149,6 +149,14 @@ int mi_reduce_sgd_raw(float* W, const float* G, size_t n, size_t replica_stride,
 int mi_reduce_sgd_bf16_raw(float* W, void* W_bf16, const float* G, size_t n, size_t replica_stride,
                            int R, float lr, void* stream);
 
+/* Same for one dense weight matrix W [rows x cols], additionally writing the transposed bf16 copy
+ * Wt_bf16 [cols x rows] in the same pass (the operand of the bf16 input-gradient GEMM) -- the GPU
+ * form of the reference forwarding each updated chunk to its consumers inside the update pass
+ * (mlp_omp.cc:240-252).  rows and cols multiples of 64 with 16-byte aligned pointers run as one
+ * tiled kernel; anything else as the flat update followed by a transpose. */
+int mi_reduce_sgd_bf16t_raw(float* W, void* W_bf16, void* Wt_bf16, const float* G, int rows, int cols,
+                            size_t replica_stride, int R, float lr, void* stream);
+
 /*
  * bf16 variants of the three GEMMs (bf16 stored as 16-bit words, fp32 accumulation on
  * v_mfma_f32_32x32x16_bf16).  A bf16 MFMA reads 8 consecutive k per lane, so every operand must be

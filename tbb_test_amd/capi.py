@@ -45,6 +45,7 @@ SIGNATURES = {
                     c_void_p, c_longlong, c_void_p],
     "mi_reduce_sgd_raw": [c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_float, c_void_p],
     "mi_reduce_sgd_bf16_raw": [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_float, c_void_p],
+    "mi_reduce_sgd_bf16t_raw": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_size_t, c_int, c_float, c_void_p],
     "mi_hgemm_nt": [c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
     "mi_hgemm_nn": [c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
     "mi_hgemm_tn": [c_int, c_int, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_int, c_longlong, c_void_p,

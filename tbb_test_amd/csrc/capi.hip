@@ -312,25 +312,41 @@ int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
 }
 
 int op_update(mi_mlp* h, int l_or_all, float lr, hipStream_t s) {
-  size_t off = 0, n = h->stride;
-  int layer_slot = 0;
-  if (l_or_all >= 0) {
-    off = h->woff[l_or_all];
-    n = (l_or_all + 1 < h->L ? h->woff[l_or_all + 1] : h->stride) - off;
-    layer_slot = l_or_all;
-  }
-  TimedScope ts(h, s, MI_WGT_UPDATE, l_or_all >= 0 ? layer_slot : -1);
+  TimedScope ts(h, s, MI_WGT_UPDATE, l_or_all >= 0 ? l_or_all : -1);
   if (ts.status) return ts.status;
-  hipError_t e = mi::reduce_sgd(h->params + off, h->params16 ? h->params16 + off : nullptr, h->grads + off, n,
-                                h->stride, h->R, lr, s, h->neg_lr_dev);
-  if (e != hipSuccess) return hip_fail(e, "reduce+SGD launch");
-  if (h->params16T) {  // refresh the transposed bf16 weight copies the input-gradient GEMMs read
-    const int first = l_or_all >= 0 ? l_or_all : 0, last = l_or_all >= 0 ? l_or_all : h->L - 1;
-    for (int l = first; l <= last && e == hipSuccess; ++l)
-      e = mi::transpose_bf16(1, h->nf[l + 1], h->nf[l], h->params16 + h->woff[l], h->nf[l], 0,
-                             h->params16T + h->woff[l], h->nf[l + 1], 0, s);
-    if (e != hipSuccess) return hip_fail(e, "weight transpose launch");
+  hipError_t e = hipSuccess;
+  if (!h->params16T) {
+    // fp32 model: one flat launch over the layer's segment (W_l | b_l) or over the whole arena
+    size_t off = 0, n = h->stride;
+    if (l_or_all >= 0) {
+      off = h->woff[l_or_all];
+      n = (l_or_all + 1 < h->L ? h->woff[l_or_all + 1] : h->stride) - off;
+    }
+    e = mi::reduce_sgd(h->params + off, nullptr, h->grads + off, n, h->stride, h->R, lr, s, h->neg_lr_dev);
+    if (e != hipSuccess) return hip_fail(e, "reduce+SGD launch");
+    return ts.finish();
   }
+  // bf16 model, per layer: W_l with both bf16 copies (W for the forward GEMM, W^T for the
+  // input-gradient GEMM) written in the same pass, the bias segment by extra workgroups of the same launch.
+  // Shapes the tiled kernel cannot take use the flat kernel and a transpose launch.
+  const int first = l_or_all >= 0 ? l_or_all : 0, last = l_or_all >= 0 ? l_or_all : h->L - 1;
+  for (int l = first; l <= last && e == hipSuccess; ++l) {
+    const size_t wo = h->woff[l], bo = h->boff[l];
+    const size_t seg_end = l + 1 < h->L ? h->woff[l + 1] : h->stride;
+    const int rows = h->nf[l + 1], cols = h->nf[l];
+    if (mi::reduce_sgd_tiled_fits(h->params + wo, h->params16 + wo, h->params16T + wo, h->grads + wo, rows, cols,
+                                  h->stride, seg_end - bo, h->R)) {
+      // the arena pads W_l to 64 floats, and rows * cols is a multiple of 64 here: b_l follows W_l directly
+      e = mi::reduce_sgd_tiled(h->params + wo, h->params16 + wo, h->params16T + wo, h->grads + wo, rows, cols,
+                               h->stride, seg_end - bo, h->R, lr, s, h->neg_lr_dev);
+    } else {
+      e = mi::reduce_sgd(h->params + wo, h->params16 + wo, h->grads + wo, seg_end - wo, h->stride, h->R, lr, s,
+                         h->neg_lr_dev);
+      if (e == hipSuccess)
+        e = mi::transpose_bf16(1, rows, cols, h->params16 + wo, cols, 0, h->params16T + wo, rows, 0, s);
+    }
+  }
+  if (e != hipSuccess) return hip_fail(e, "reduce+SGD launch");
   return ts.finish();
 }
 
@@ -701,6 +717,27 @@ int mi_reduce_sgd_bf16_raw(float* W, void* W_bf16, const float* G, size_t n, siz
   MI_REQUIRE(R == 1 || replica_stride >= n, "replica_stride %zu < n %zu", replica_stride, n);
   hipError_t e = mi::reduce_sgd(W, (uint16_t*)W_bf16, G, n, replica_stride, R, lr, as_stream(stream));
   if (e != hipSuccess) return hip_fail(e, "mi_reduce_sgd_bf16_raw launch");
+  return MI_OK;
+}
+
+int mi_reduce_sgd_bf16t_raw(float* W, void* W_bf16, void* Wt_bf16, const float* G, int rows, int cols,
+                            size_t replica_stride, int R, float lr, void* stream) {
+  MI_REQUIRE(R >= 1, "R must be at least 1 (got %d)", R);
+  MI_REQUIRE(rows >= 0 && cols >= 0, "negative size");
+  if (rows == 0 || cols == 0) return MI_OK;
+  MI_REQUIRE(W && G && W_bf16 && Wt_bf16, "null pointer");
+  const size_t n = (size_t)rows * cols;
+  MI_REQUIRE(R == 1 || replica_stride >= n, "replica_stride %zu < rows * cols %zu", replica_stride, n);
+  hipStream_t s = as_stream(stream);
+  hipError_t e;
+  if (mi::reduce_sgd_tiled_fits(W, (uint16_t*)W_bf16, (uint16_t*)Wt_bf16, G, rows, cols, replica_stride, 0, R)) {
+    e = mi::reduce_sgd_tiled(W, (uint16_t*)W_bf16, (uint16_t*)Wt_bf16, G, rows, cols, replica_stride, 0, R, lr, s);
+  } else {  // any shape: flat update, then a transpose of the bf16 copy
+    e = mi::reduce_sgd(W, (uint16_t*)W_bf16, G, n, replica_stride, R, lr, s);
+    if (e == hipSuccess)
+      e = mi::transpose_bf16(1, rows, cols, (const uint16_t*)W_bf16, cols, 0, (uint16_t*)Wt_bf16, rows, 0, s);
+  }
+  if (e != hipSuccess) return hip_fail(e, "mi_reduce_sgd_bf16t_raw launch");
   return MI_OK;
 }
 

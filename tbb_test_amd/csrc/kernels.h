@@ -88,6 +88,17 @@ hipError_t colsum_f32(int R, int M, int K, const float* A, int lda, float* out, 
 hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t stride, int R, float lr,
                       hipStream_t s, const float* neg_lr_dev = nullptr);
 
+// Same update for one weight matrix W [rows x cols] (dense) of a bf16 model, writing the bf16 copy
+// W16 [rows x cols] and the transposed bf16 copy W16T [cols x rows] in the same pass; the `tail`
+// floats that follow the matrix in W, W16 and every replica of G (a layer's bias and padding) are
+// updated the flat way by the same launch.  Needs rows and cols multiples of 64, tail a multiple
+// of 4 and 16-byte aligned pointers (reduce_sgd_tiled_fits); `stride` = floats between consecutive
+// replicas' gradients.
+bool reduce_sgd_tiled_fits(const float* W, const uint16_t* W16, const uint16_t* W16T, const float* G, int rows,
+                           int cols, size_t stride, size_t tail, int R);
+hipError_t reduce_sgd_tiled(float* W, uint16_t* W16, uint16_t* W16T, const float* G, int rows, int cols, size_t stride,
+                            size_t tail, int R, float lr, hipStream_t s, const float* neg_lr_dev = nullptr);
+
 // bf16: C = A[M,K] * B[N,K]^T with fp32 accumulation, both operands K-contiguous, blockIdx.z
 // batches with element strides batchA/B/C.  out_kind: 0 fp32 plain, 1 bf16 with bias + optional
 // ReLU, 2 bf16 zeroed where mask (bf16) <= 0, 3 bf16 plain.  Ct (bf16 output kinds, batch 1): the

@@ -137,6 +137,28 @@ def test_reduce_sgd_writes_bf16_copy():
     assert np.array_equal(d16.to_numpy((n,), np.uint16), to_bf16_bits(want))
 
 
+@pytest.mark.parametrize("rows,cols", [(128, 192), (64, 64), (512, 320), (128, 512), (192, 256), (100, 70), (64, 72)])
+@pytest.mark.parametrize("R", [1, 3, 4])
+def test_reduce_sgd_writes_both_bf16_copies_in_one_pass(rows, cols, R):
+    """The update of one weight matrix with the bf16 copy and the transposed bf16 copy (tiled kernel
+    for multiples of 64, flat kernel + transpose otherwise): fp32 result bit-exact against the
+    oracle, both copies equal to its rounding; replica stride larger than the matrix."""
+    rng = np.random.default_rng(rows + cols + R)
+    n, stride = rows * cols, rows * cols + 256
+    W = rng.uniform(-1, 1, n).astype(np.float32)
+    G = rng.standard_normal((R, stride)).astype(np.float32)
+    dW, dG = capi.DeviceBuffer.from_numpy(W), capi.DeviceBuffer.from_numpy(G)
+    d16, d16t = capi.DeviceBuffer(n * 2), capi.DeviceBuffer(n * 2)
+    capi.check(capi.lib().mi_reduce_sgd_bf16t_raw(dW.ptr, d16.ptr, d16t.ptr, dG.ptr, rows, cols, stride, R,
+                                                  ctypes.c_float(0.01), None))
+    capi.check(capi.lib().mi_stream_sync(None))
+    want = oracle.reduce_sgd(W, G[:, :n], 0.01)
+    assert np.array_equal(dW.to_numpy((n,)).view(np.uint32), want.view(np.uint32))
+    want16 = to_bf16_bits(want).reshape(rows, cols)
+    assert np.array_equal(d16.to_numpy((rows, cols), np.uint16), want16)
+    assert np.array_equal(d16t.to_numpy((cols, rows), np.uint16), want16.T)
+
+
 LR = 0.01
 STEP_CONFIGS = {
     "square": ([256, 256, 256, 256], 128, 2),
