@@ -357,15 +357,28 @@ __global__ __launch_bounds__(256) void mask_copy_kernel(float* __restrict__ dst,
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step)
     dst[i] = act[i] > 0.0f ? g[i] : 0.0f;
 }
+// the same on bf16 words: positive = sign bit clear and not zero (a NaN output keeps the gradient,
+// as the fp32 comparison drops it; outputs of the forward GEMM are finite)
+__global__ __launch_bounds__(256) void mask_copy_bf16_kernel(uint16_t* __restrict__ dst, const uint16_t* __restrict__ g,
+                                                             const uint16_t* __restrict__ act, size_t n) {
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step) {
+    const float a = __uint_as_float((unsigned)act[i] << 16);
+    dst[i] = a > 0.0f ? g[i] : (uint16_t)0;
+  }
+}
 
 int op_last_mask(mi_mlp* h, hipStream_t s) {
   if (!(h->flags & MI_FLAG_RELU_LAST)) return MI_OK;
-  if (h->dtype != MI_F32) return fail(MI_ERR_UNSUPPORTED, "bf16 ReLU-last is not implemented in this build");
   const size_t n = (size_t)h->MB * h->nf[h->L];
   size_t blocks = (n + 255) / 256;
   if (blocks > 4096) blocks = 4096;
-  mi::launch_kernel(mask_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float*)h->dz[(h->L - 1) % h->ndz],
-                     (const float*)h->dy, (const float*)h->acts[h->L], n);
+  if (h->dtype == MI_F32)
+    mi::launch_kernel(mask_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float*)h->dz[(h->L - 1) % h->ndz],
+                      (const float*)h->dy, (const float*)h->acts[h->L], n);
+  else
+    mi::launch_kernel(mask_copy_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, s,
+                      (uint16_t*)h->dz[(h->L - 1) % h->ndz], (const uint16_t*)h->dy, (const uint16_t*)h->acts[h->L], n);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e, "mask launch");
   return MI_OK;
@@ -846,8 +859,6 @@ int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_repli
   MI_REQUIRE((long long)batch_per_replica * R <= 0x7fffffffLL, "R * batch overflows int");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "unknown dtype %d", dtype);
   for (int l = 0; l <= L; ++l) MI_REQUIRE(nfeatures[l] >= 1, "nfeatures[%d] = %d must be positive", l, nfeatures[l]);
-  if (dtype == MI_BF16 && (flags & MI_FLAG_RELU_LAST))
-    return fail(MI_ERR_UNSUPPORTED, "MI_FLAG_RELU_LAST is not implemented for bf16 models");
 
   int count = 0;
   if (hipGetDeviceCount(&count) != hipSuccess || count == 0) return fail(MI_ERR_NO_DEVICE, "no HIP device visible");

@@ -54,6 +54,8 @@ struct HGemmArgs {
   // per group -- the K-contiguous per-replica copy the weight-gradient GEMM reads
   u16* Ct;
   int ct_rows;
+  // guarded instances: whether A / B may be read with 16-byte vector loads
+  int vec_a, vec_b;
 };
 
 __device__ __forceinline__ u16 f2bf(float f) {
@@ -110,7 +112,9 @@ __device__ __forceinline__ void tile_of_workgroup(int id, int tiles_m, int tiles
 // `mask_ld` elements per row; (row_l, col_l) is this wavefront's first row / column inside it.
 // MASK_LDS is a template argument, not a test of mask_lds inside the loops: a pointer that may be
 // either LDS or global memory turns every mask read into a flat load behind a branch.
-template <int TM, int TN, int EPI, bool MASK_LDS = false>
+// GUARD: the tile may stick out of C; rows >= p.M and columns >= p.N are skipped (and neither bias
+// nor mask is read there).  Guarded instances have no transposed second output.
+template <int TM, int TN, int EPI, bool MASK_LDS = false, bool GUARD = false>
 __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[TM][TN], int row0, int colw, int l32,
                                              int hi, u16* lds = nullptr, const u16* mask_lds = nullptr, int mask_ld = 0,
                                              int row_l = 0, int col_l = 0) {
@@ -118,7 +122,8 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
   const int col0 = colw + l32;
   float bias_v[TN];
 #pragma unroll
-  for (int j = 0; j < TN; ++j) bias_v[j] = (EPI == EPH_BIAS_RELU && p.bias) ? p.bias[col0 + j * 32] : 0.0f;
+  for (int j = 0; j < TN; ++j)
+    bias_v[j] = (EPI == EPH_BIAS_RELU && p.bias && (!GUARD || col0 + j * 32 < p.N)) ? p.bias[col0 + j * 32] : 0.0f;
   float* __restrict__ cf = reinterpret_cast<float*>(p.C) + (size_t)blockIdx.z * p.batchC;
   u16* __restrict__ ch = reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC;
   unsigned pk[TM][TN][8];  // bf16 results, two rows per register: (4g, 4g+1) and (4g+2, 4g+3)
@@ -130,8 +135,10 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = row0 + i * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
+        if (GUARD && row >= p.M) continue;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) cf[(size_t)row * p.ldc + col0 + j * 32] = acc[i][j][r];
+        for (int j = 0; j < TN; ++j)
+          if (!GUARD || col0 + j * 32 < p.N) cf[(size_t)row * p.ldc + col0 + j * 32] = acc[i][j][r];
       }
     return;
   } else {
@@ -148,6 +155,8 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
           const int col = col0 + j * 32;
+          if (GUARD && (col >= p.N || row >= p.M)) continue;
+          const bool second_row = !GUARD || row + 1 < p.M;
           f32x2_t v = {acc[i][j][2 * rp], acc[i][j][2 * rp + 1]};
           if (EPI == EPH_BIAS_RELU) {
             v[0] += bias_v[j];
@@ -165,7 +174,7 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
                 mk = reinterpret_cast<lds_u16*>(
                     (__attribute__((address_space(3))) const char*)(size_t)mask_lds_addr)[(row + e - row0 + row_l) * mask_ld + col_l + l32 + j * 32];
               } else {
-                mk = p.mask[(size_t)(row + e) * p.ldmask + col];
+                mk = (e == 0 || second_row) ? p.mask[(size_t)(row + e) * p.ldmask + col] : (u16)0;
               }
               if (!(bf2f(mk) > 0.0f)) v[e] = 0.0f;
             }
@@ -173,12 +182,12 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
           const unsigned two = __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
           pk[i][j][rp] = two;
           ch[(size_t)row * p.ldc + col] = (u16)two;
-          ch[(size_t)(row + 1) * p.ldc + col] = (u16)(two >> 16);
+          if (second_row) ch[(size_t)(row + 1) * p.ldc + col] = (u16)(two >> 16);
         }
       }
     }
   }
-  if (EPI == EPH_F32 || !p.Ct) return;
+  if (EPI == EPH_F32 || GUARD || !p.Ct) return;
   if (MASK_LDS && lds) __syncthreads();  // the staging regions overlap the mask tile other wavefronts still read
   // the tile lies inside one row group: ct_rows is a multiple of the tile height
   const int group = row0 / p.ct_rows, m_local0 = row0 - group * p.ct_rows;
@@ -229,9 +238,14 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
 // written to LDS at its end, barrier at the step boundary) -- what fits when BK = 64 makes a
 // 256 x 256 tile 72 KB per buffer.  BK = 64 matters for bandwidth: a tile row is then one whole
 // 128-byte cache line, where BK = 32 touches half a line per row and step.
-template <int BM, int BN, int BK, int WM, int WN, int EPI, int PF = 1, int STAGES = 3>
+// GUARD = true: M, N, K need not be multiples of the tile and nothing need be aligned: a tile's
+// loads outside the operands read zero (whole 16-byte pieces where p.vec_a / p.vec_b say that the
+// operand's alignment allows vector loads and the piece lies inside K, element by element
+// otherwise), and the epilogue skips what lies outside C.
+template <int BM, int BN, int BK, int WM, int WN, int EPI, int PF = 1, int STAGES = 3, bool GUARD = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
   static_assert(PF >= 1 && PF <= 3, "prefetch distance");
+  static_assert(!GUARD || (STAGES == 3 && PF == 1), "the guarded loads are written for the three-buffer loop");
   static_assert(STAGES == 3 || (STAGES == 2 && PF == 1), "two buffers only with the plain schedule");
   constexpr int NT = WM * WN * 64;
   constexpr int WTM = BM / WM, WTN = BN / WN;
@@ -269,7 +283,34 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   u32x4 ra[PF][NVA], rb[PF][NVB];
+  int k_next = 0;  // GUARD: first k of the next tile to fetch
+  // one 16-byte piece (8 consecutive k of one row) that may lie partly or wholly outside the operand
+  auto piece = [&](const u16* row_ptr, bool row_ok, int k, bool vec) {
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (!row_ok || k >= p.K) return v;
+    if (vec && k + 8 <= p.K) return *reinterpret_cast<const u32x4*>(row_ptr + k);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const unsigned x = (k + e < p.K) ? (unsigned)row_ptr[k + e] : 0u;
+      v[e >> 1] |= x << ((e & 1) * 16);
+    }
+    return v;
+  };
   auto fetch = [&](u32x4 (&sa)[NVA], u32x4 (&sb)[NVB]) {
+    if constexpr (GUARD) {
+#pragma unroll
+      for (int i = 0; i < NVA; ++i) {
+        const int idx = tid + i * NT, row = idx / VPR, c = idx % VPR;
+        sa[i] = piece(a_ptr + (size_t)row * p.lda, m0 + row < p.M, k_next + c * 8, p.vec_a);
+      }
+#pragma unroll
+      for (int i = 0; i < NVB; ++i) {
+        const int idx = tid + i * NT, row = idx / VPR, c = idx % VPR;
+        sb[i] = piece(b_ptr + (size_t)row * p.ldb, n0 + row < p.N, k_next + c * 8, p.vec_b);
+      }
+      k_next += BK;
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NVA; ++i) {
       const int idx = tid + i * NT, row = idx / VPR, c = idx % VPR;
@@ -315,7 +356,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
     }
   };
 
-  const int nk = p.K / BK;
+  const int nk = GUARD ? (p.K + BK - 1) / BK : p.K / BK;
   fetch(ra[0], rb[0]);
   stash(0, ra[0], rb[0]);
   if constexpr (STAGES == 2) {
@@ -373,7 +414,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
   }
   }
 
-  store_tile_h<TM, TN, EPI>(p, acc, m0 + wm0, n0 + wn0, l32, hi);
+  store_tile_h<TM, TN, EPI, false, GUARD>(p, acc, m0 + wm0, n0 + wn0, l32, hi);
 }
 
 // ---- the same GEMM with direct global -> LDS loads ------------------------------------------------
@@ -677,7 +718,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
   else store_tile_h<TM, TN, EPI, false>(p, acc, m0 + wm0, n0 + wn0, l32, hi, stage, nullptr, BN, wm0, wn0);
 }
 
-// Any-shape fallback: one thread per output element, fp32 accumulation in k order.
+// Fallback for an empty contraction (K = 0) and for forced variants that do not fit: one thread per
+// output element, fp32 accumulation in k order.
 template <int EPI>
 __global__ __launch_bounds__(256) void gemm_bf16_generic(HGemmArgs p) {
   const int col = blockIdx.x * 16 + (threadIdx.x & 15), row = blockIdx.y * 16 + (threadIdx.x >> 4);
@@ -699,15 +741,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_generic(HGemmArgs p) {
   (reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC)[(size_t)row * p.ldc + col] = f2bf(v);
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int EPI, int PF = 1, int STAGES = 3>
+template <int BM, int BN, int BK, int WM, int WN, int EPI, int PF = 1, int STAGES = 3, bool GUARD = false>
 static hipError_t launch_h(HGemmArgs& p, int batch, hipStream_t s) {
   constexpr size_t lds_bytes = STAGES * (size_t)(BM + BN) * BK * sizeof(u16);
   static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB of LDS");
-  auto kern = gemm_bf16_mfma<BM, BN, BK, WM, WN, EPI, PF, STAGES>;
+  auto kern = gemm_bf16_mfma<BM, BN, BK, WM, WN, EPI, PF, STAGES, GUARD>;
   static LdsOptIn opt_in;
   if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) return e;
-  p.tiles_m = p.M / BM;
-  p.tiles_n = p.N / BN;
+  p.tiles_m = GUARD ? (p.M + BM - 1) / BM : p.M / BM;
+  p.tiles_n = GUARD ? (p.N + BN - 1) / BN : p.N / BN;
   launch_kernel(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WM * WN * 64), lds_bytes, s, p);
   return hipGetLastError();
 }
@@ -746,11 +788,15 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     else if (fits(256, 256, 32) && t256 >= 256) variant = 13;
     else if (fits(128, 128, 32) && (long long)(p.M / 128) * (p.N / 128) * batch >= 128) variant = 3;
     else if (fits(64, 64, 32)) variant = 5;
+    else if (p.K > 0)  // ragged shape or unaligned storage: the guarded MFMA instances
+      variant = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * batch >= 192 ? 21 : 22;
     else variant = -1;
   }
+  p.vec_a = al16(p.A) && p.lda % 8 == 0 && p.batchA % 8 == 0;
+  p.vec_b = al16(p.B) && p.ldb % 8 == 0 && p.batchB % 8 == 0;
   {  // the tile height decides whether the transposed output is possible; if not, drop it
     const int bm = (variant == 3 || variant == 17) ? 128 : variant == 5 ? 64 : 256;
-    if (want_ct && (EPI == EPH_F32 || !ct_ok(bm))) {
+    if (want_ct && (EPI == EPH_F32 || variant == 21 || variant == 22 || !ct_ok(bm))) {
       p.Ct = nullptr;
       if (wrote_ct) *wrote_ct = false;
     }
@@ -762,6 +808,8 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     case 13: if (fits(256, 256, 32)) return launch_dma<256, 256, 32, 2, 4, EPI, 4>(p, batch, s); break;
     case 17: if (fits(128, 128, 32)) return launch_dma<128, 128, 32, 2, 2, EPI, 4>(p, batch, s); break;
     case 19: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2>(p, batch, s); break;
+    case 21: if (p.K > 0) return launch_h<128, 128, 32, 2, 2, EPI, 1, 3, true>(p, batch, s); break;
+    case 22: if (p.K > 0) return launch_h<64, 64, 32, 2, 2, EPI, 1, 3, true>(p, batch, s); break;
     default: break;
   }
   if (wrote_ct) *wrote_ct = false;  // the any-shape kernel has no transposed output

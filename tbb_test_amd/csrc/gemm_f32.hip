@@ -1108,6 +1108,9 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
 
 hipError_t sgemm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
                     int ldc, const float* bias, int relu, hipStream_t s, int variant) {
+  // automatic choice: a layer of at most SKINNY_MAX outputs is matrix-vector work
+  if ((variant == 0 || variant == 100) && N <= SKINNY_MAX && K > 0)
+    return sgemv_nt(M, N, K, A, lda, B, ldb, C, ldc, bias, relu, s);
   GemmArgs p{};
   p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.bias = bias; p.relu = relu;
@@ -1116,6 +1119,8 @@ hipError_t sgemm_nt(int M, int N, int K, const float* A, int lda, const float* B
 
 hipError_t sgemm_nn(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
                     int ldc, const float* mask, int ldmask, hipStream_t s, int variant) {
+  if ((variant == 0 || variant == 100) && K <= SKINNY_MAX && K > 0)
+    return sgemv_nn(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, s);
   GemmArgs p{};
   p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.mask = mask; p.ldmask = ldmask;
@@ -1126,6 +1131,8 @@ hipError_t sgemm_nn(int M, int N, int K, const float* A, int lda, const float* B
 hipError_t sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const float* B, int ldb,
                     float* C, int ldc, long long strideC, float* colsum, long long stride_colsum,
                     hipStream_t s, int variant) {
+  if (variant == 0 && M <= SKINNY_MAX && K > 0)
+    return sgemv_tn(R, M, N, K, A, lda, B, ldb, C, ldc, strideC, colsum, stride_colsum, s);
   GemmArgs p{};
   p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.batchA = (long long)K * lda;  // replica r reads rows [r*K, (r+1)*K) of both operands

@@ -78,6 +78,17 @@ hipError_t sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const f
                     float* C, int ldc, long long strideC, float* colsum, long long stride_colsum,
                     hipStream_t s, int variant);
 
+// gemv_f32.hip: the same three operations for layers whose output width is at most SKINNY_MAX
+// (N of the forward GEMM, M of the weight gradient, K of the input gradient), as matrix-vector
+// passes at memory speed.  Any alignment; the automatic choice of sgemm_* takes them.
+constexpr int SKINNY_MAX = 16;
+hipError_t sgemv_nt(int M, int N, int K, const float* X, int ldx, const float* W, int ldw, float* Y, int ldy,
+                    const float* bias, int relu, hipStream_t s);
+hipError_t sgemv_tn(int R, int M, int N, int K, const float* dZ, int lddz, const float* A, int lda, float* dW,
+                    int lddw, long long strideW, float* colsum, long long stride_colsum, hipStream_t s);
+hipError_t sgemv_nn(int M, int N, int K, const float* dZ, int lddz, const float* W, int ldw, float* dA, int ldda,
+                    const float* mask, int ldmask, hipStream_t s);
+
 // out[r*stride_out + j] = sum_{i in [r*K, (r+1)*K)} A[i*lda + j], j in [0, M)
 hipError_t colsum_f32(int R, int M, int K, const float* A, int lda, float* out, long long stride_out,
                       hipStream_t s);

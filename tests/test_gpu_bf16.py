@@ -56,7 +56,7 @@ HSHAPES = [(64, 64, 32), (128, 128, 64), (256, 256, 96), (512, 256, 128), (256, 
            # K loops of the direct-load kernels: one step, and every length of the conditional tail after
            # the branch-free turns of the ring (two buffers at BK = 64, four at BK = 32)
            (256, 256, 64), (256, 256, 192), (256, 256, 320), (256, 256, 448)]
-HVARIANTS = [0, 3, 4, 5, 13, 17, 19]
+HVARIANTS = [0, 3, 4, 5, 13, 17, 19, 21, 22]   # 21, 22: the guarded any-shape MFMA instances
 
 
 @pytest.mark.parametrize("variant", HVARIANTS)
@@ -86,6 +86,30 @@ def test_hgemm_forward_and_input_gradient(shape, variant):
         assert np.all(got[act <= 0] == 0.0)
     finally:
         lib.mi_set_hgemm_variant(0)
+
+
+@pytest.mark.parametrize("shape", [(130, 70, 100), (64, 64, 64), (33, 200, 17)])
+def test_hgemm_on_operands_that_allow_no_vector_access(shape):
+    """Operands that start one element past a 16-byte boundary, with leading dimensions that are
+    not multiples of 8: the guarded MFMA instances read them element by element."""
+    M, N, K = shape
+    rng = np.random.default_rng(M * N + K)
+    lda, ldb, ldc = K + 3, K + 5, N + 1
+    A = bf16_round(rng.uniform(-1, 1, (M, lda)))
+    B = bf16_round(rng.uniform(-1, 1, (N, ldb)))
+    bias = rng.uniform(-1, 1, N).astype(np.float32)
+    lib = capi.lib()
+    pad = np.zeros(1, np.uint16)
+    dA = capi.DeviceBuffer.from_numpy(np.concatenate([pad, to_bf16_bits(A).ravel()]))
+    dB = capi.DeviceBuffer.from_numpy(np.concatenate([pad, to_bf16_bits(B).ravel()]))
+    dbias = capi.DeviceBuffer.from_numpy(bias)
+    dC = capi.DeviceBuffer((1 + M * ldc) * 2)
+    dC.zero()
+    capi.check(lib.mi_hgemm_nt(M, N, K, dA.ptr + 2, lda, dB.ptr + 2, ldb, dC.ptr + 2, ldc, dbias.ptr, 0, None))
+    capi.check(lib.mi_stream_sync(None))
+    out = from_bf16_bits(dC.to_numpy((1 + M * ldc,), np.uint16))[1:].reshape(M, ldc)
+    assert rel_err(out[:, :N], oracle.fc_forward(A[:, :K], B[:, :K], bias, False)) <= 4e-3
+    assert np.all(out[:, N:] == 0)   # nothing written between the rows of C
 
 
 @pytest.mark.parametrize("variant", HVARIANTS)
@@ -177,13 +201,14 @@ def _check_bf16_step(nf, B, R, flags, seed=31, expect_fused=None):
         h.set_weights(l, Ws[l], bs[l])
     h.set_input(X)
     h.set_dy(dY)
-    for _ in range(2 if flags == 0 else 1):   # with graphs: the second call is the replay
+    for _ in range(1 if flags & capi.FLAG_NO_GRAPH else 2):   # with graphs: the second call is the replay
         h.snapshot_weights() if _ == 0 else h.restore_weights()
         h.step(LR)
     h.sync()
     if expect_fused is not None:  # the transposed operand copies came out of the GEMM epilogues, not a fallback
         assert h.schedule()["fused_transposes"] == expect_fused
-    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR)
+    relu_last = bool(flags & capi.FLAG_RELU_LAST)
+    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR, relu_last=relu_last)
     acts = [h.activation(l) for l in range(L + 1)]
     for l in range(L + 1):
         assert rel_err(acts[l], ref.acts[l]) <= BF16_TOL, f"activation {l}"
@@ -194,7 +219,7 @@ def _check_bf16_step(nf, B, R, flags, seed=31, expect_fused=None):
     flipped = sum(int(np.count_nonzero((acts[l] > 0) != (ref.acts[l] > 0))) for l in range(1, L))
     total = sum(acts[l].size for l in range(1, L))
     assert flipped <= 0.03 * total, f"{flipped} of {total} masks differ"
-    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR, given_acts=acts)
+    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR, given_acts=acts, relu_last=relu_last)
     assert rel_err(h.dx(), ref.dX) <= BF16_TOL
     for l in range(L):
         for r in range(R):
@@ -206,7 +231,8 @@ def _check_bf16_step(nf, B, R, flags, seed=31, expect_fused=None):
 
 
 @pytest.mark.parametrize("name", list(STEP_CONFIGS))
-@pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, 0, capi.FLAG_PER_LAYER_UPDATE])
+@pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, 0, capi.FLAG_PER_LAYER_UPDATE,
+                                   capi.FLAG_NO_GRAPH | capi.FLAG_RELU_LAST, capi.FLAG_RELU_LAST | capi.FLAG_PER_LAYER_UPDATE])
 def test_bf16_step_matches_fp32_oracle(name, flags):
     nf, B, R = STEP_CONFIGS[name]
     _check_bf16_step(nf, B, R, flags)

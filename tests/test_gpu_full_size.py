@@ -26,12 +26,17 @@ def build(nf, B, R, seed, dtype=capi.MI_F32, flags=0):
     return h, X, Ws, dY
 
 
-@pytest.mark.parametrize("name,nf,B,R", [("C3", [4096] * 5, 2048, 2), ("C4", [2048] * 21, 256, 8)])
+@pytest.mark.parametrize("name,nf,B,R", [("C3", [4096] * 5, 2048, 2), ("C4", [2048] * 21, 256, 8),
+                                         # the reference's own default model (mlp_bench_common.h:26): last layer 1024 -> 1
+                                         ("ref", [1024] * 7 + [1], 1024, 4)])
 def test_fp32_config_full_size(name, nf, B, R):
     L = len(nf) - 1
-    h, X, Ws, dY = build(nf, B, R, seed=7)
+    h, X, Ws, dY = build(nf, B, R, seed=7, flags=capi.FLAG_PER_LAYER_UPDATE)
+    h.snapshot_weights()
+    for _ in range(2):              # the second step replays the captured graph
+        h.restore_weights()
+        h.step(LR)
     bs = [np.zeros(n, np.float32) for n in nf[1:]]
-    h.step(LR)
     h.sync()
     acts = [h.activation(l) for l in range(L + 1)]
     ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR)
