@@ -276,7 +276,11 @@ int mi_mlp_get_weight_shadow(mi_mlp* h, int l, int transposed, float* dst, int l
  *   info[2]  1 = steps replay a captured HIP graph
  *   info[3]  bf16 models: how many of the 2(L-1) transposed operand copies of the weight-gradient
  *            GEMMs were written by the epilogue of the GEMM that produced the operand (the rest
- *            came from separate transpose launches); 0 for fp32 models */
+ *            came from separate transpose launches); 0 for fp32 models
+ *   info[4]  1 = small fp32 model: weight gradient and input gradient of a layer share one launch,
+ *            everything on one stream with one update launch (fewest launches; the scheduling
+ *            flags have nothing to overlap there)
+ * info must have room for 5 ints. */
 int mi_mlp_get_schedule(mi_mlp* h, int* info);
 
 /* Number of parameters P = sum_l (N_l*N_{l+1} + N_{l+1}) and the padded element stride between
@@ -337,7 +341,8 @@ int mi_l2_loss_static(int dtype, int R, int batch_per_replica, int N, const void
  * microseconds, loadable in a Chrome-trace viewer).  Names follow the reference's tasks
  * (mlp_tbb.cc:176-178,325-327,840,982,1104): FC_<l>_0, FCWgtGradient_<l>_0, FCBwdGradient_<l>_0;
  * the fused reduce + SGD launch of layer l is ReduceScatterAllGather_<l>_0 (_all_ when one launch
- * covers every layer), the loss kernel L2Loss_0.  pid 0 is the GPU, tid 0 / 1 the main / second
+ * covers every layer), the loss kernel L2Loss_0; small fp32 models, whose two backward GEMMs of a
+ * layer share a launch, show FCWgtGradient+FCBwdGradient_<l>_0 instead of the two.  pid 0 is the GPU, tid 0 / 1 the main / second
  * stream.  The step updates the weights like any other.
  */
 int mi_mlp_trace_step(mi_mlp* h, float lr, const char* path);

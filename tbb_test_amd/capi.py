@@ -264,11 +264,11 @@ class MlpHandle:
         return self._get(lib().mi_mlp_get_weight_shadow, shape, l, int(transposed))
 
     def schedule(self):
-        """What the last step did: dict(dual_streams, per_layer_update, graph, fused_transposes)."""
-        info = (c_int * 4)()
+        """What the last step did: dict(dual_streams, per_layer_update, graph, fused_transposes, paired_backward)."""
+        info = (c_int * 5)()
         check(lib().mi_mlp_get_schedule(self._h, info))
         return {"dual_streams": bool(info[0]), "per_layer_update": bool(info[1]), "graph": bool(info[2]),
-                "fused_transposes": int(info[3])}
+                "fused_transposes": int(info[3]), "paired_backward": bool(info[4])}
 
     def snapshot_weights(self): check(lib().mi_mlp_snapshot_weights(self._h))
     def restore_weights(self): check(lib().mi_mlp_restore_weights(self._h))

@@ -126,7 +126,7 @@ struct mi_mlp {
   float neg_lr_value = 0.0f;
   bool neg_lr_valid = false;
   // what the last enqueue_step decided (mi_mlp_get_schedule)
-  bool last_dual = false, last_per_layer = false;
+  bool last_dual = false, last_per_layer = false, last_paired = false;
 
   size_t esize() const { return dtype == MI_BF16 ? 2 : 4; }
   size_t maxw() const {
@@ -176,6 +176,7 @@ int get_event(mi_mlp* h, hipEvent_t* ev) {
 }
 
 constexpr int TRACE_LOSS = 100;   // pseudo-breakdown of the loss kernel in a timeline
+constexpr int TRACE_PAIR = 101;   // weight gradient + input gradient of a layer in one launch
 constexpr int LOSS_CHUNKS = 64;   // partial sums per replica
 
 struct TimedScope {
@@ -309,6 +310,32 @@ int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
   }
   if (e != hipSuccess) return hip_fail(e, "input-gradient GEMM launch");
   return ts.finish();
+}
+
+// Weight gradient and input gradient of layer l in one launch (small fp32 layers only, see
+// small_model()).  Booked as one weight-gradient scope in a timeline.
+int op_backward_pair(mi_mlp* h, int l, hipStream_t s) {
+  TimedScope ts(h, s, TRACE_PAIR, l);
+  if (ts.status) return ts.status;
+  float* out = (float*)((l == 0) ? h->dx : h->dz[(l - 1) % h->ndz]);
+  const float* mask = (l == 0) ? nullptr : (const float*)h->acts[l];
+  hipError_t e = mi::sgemm_backward_pair(h->R, h->MB, h->nf[l + 1], h->nf[l], (const float*)dz_of_layer(h, l),
+                                         (const float*)h->acts[l], h->params + h->woff[l], h->grads + h->woff[l],
+                                         (long long)h->stride, h->grads + h->boff[l], (long long)h->stride, out, mask, s);
+  if (e != hipSuccess) return hip_fail(e, "backward pair launch");
+  return ts.finish();
+}
+
+// A model all of whose backward GEMMs are small enough for the paired launch: its step is a chain
+// of launches of a few microseconds each, so the schedule that counts is the one with the fewest
+// launches -- one stream, weight and input gradient of a layer in one launch, one update launch.
+bool small_model(const mi_mlp* h) {
+  if (h->dtype != MI_F32) return false;
+  for (int k = 0; k < 3; ++k)
+    if (g_variant[k].load() != 0) return false;  // a forced tile configuration is honoured by the separate launches
+  for (int l = 0; l < h->L; ++l)
+    if (!mi::sgemm_backward_pair_fits(h->R, h->MB, h->nf[l + 1], h->nf[l])) return false;
+  return true;
 }
 
 int op_update(mi_mlp* h, int l_or_all, float lr, hipStream_t s) {
@@ -517,15 +544,18 @@ int enqueue_step(mi_mlp* h, float lr) {
   if ((rc = op_last_mask(h, s))) return rc;
   // While per-kernel event timing is on, everything runs back to back on one stream with one
   // update launch: durations of kernels that overlap cannot be attributed to a kernel.
-  const bool per_layer = (h->flags & MI_FLAG_PER_LAYER_UPDATE) != 0 && !h->timing;
+  // (per-kernel timing keeps the separate launches so that every phase has its own figures)
+  const bool paired = small_model(h) && !h->timing;
+  const bool per_layer = (h->flags & MI_FLAG_PER_LAYER_UPDATE) != 0 && !h->timing && !paired;
   // Two backward streams pay while a GEMM launch leaves CUs idle at its start and end, i.e. up to
   // a few tiles per CU (configs 2 and 4: 256 tiles of 128 x 128 per input-gradient launch, 3-5 %
   // faster with two streams).  GEMMs with many tiles per CU only get in each other's way (config
   // 3, 1024 tiles: 11.32 ms with one backward stream, 11.47 ms with two; config 5: 45.9 / 47.1 ms).
   const bool crowded = (long long)(h->MB / 128) * (long long)(h->maxw() / 128) >= 1024;
-  const bool dual = !(h->flags & MI_FLAG_SERIAL_BACKWARD) && !h->timing && !crowded;
+  const bool dual = !(h->flags & MI_FLAG_SERIAL_BACKWARD) && !h->timing && !crowded && !paired;
   h->last_dual = dual;
   h->last_per_layer = per_layer;
+  h->last_paired = paired;
   hipStream_t s2 = dual ? h->stream2 : s;
   if (dual) {  // fork: dZ_{L-1} and all activations are ready
     MI_HIP(hipEventRecord(h->ev_fork, s));
@@ -543,6 +573,10 @@ int enqueue_step(mi_mlp* h, float lr) {
   } corun_scope(h);
   const bool corun_cfg = !(h->flags & MI_FLAG_SERIAL_BACKWARD) && !crowded;
   for (int l = h->L - 1; l >= 0; --l) {
+    if (paired) {
+      if ((rc = op_backward_pair(h, l, s))) return rc;
+      continue;
+    }
     h->corun = corun_cfg && h->B < 512;
     if ((rc = op_wgrad(h, l, s2, true))) return rc;
     if (dual) {
@@ -1131,6 +1165,7 @@ int mi_mlp_trace_step(mi_mlp* h, float lr, const char* path) {
       }
       char name[64];
       if (t.breakdown == TRACE_LOSS) snprintf(name, sizeof name, "L2Loss_0");
+      else if (t.breakdown == TRACE_PAIR) snprintf(name, sizeof name, "FCWgtGradient+FCBwdGradient_%d_0", t.layer);
       else if (t.layer < 0) snprintf(name, sizeof name, "%s_all_0", kNames[t.breakdown]);
       else snprintf(name, sizeof name, "%s_%d_0", kNames[t.breakdown], t.layer);
       fprintf(f, "{\n \"ts\": %.3f,\n \"pid\": 0,\n \"tid\": %d,\n \"name\": \"%s\",\n \"ph\": \"B\"\n},\n", t0 * 1e3,
@@ -1294,6 +1329,7 @@ int mi_mlp_get_schedule(mi_mlp* h, int* info) {
     for (int l = 0; l + 1 < h->L; ++l) fused += h->dzT_fused[l % h->ndz] ? 1 : 0;  // dZ_l^T written by dgrad(l+1)
   }
   info[3] = fused;
+  info[4] = h->last_paired ? 1 : 0;
   return MI_OK;
 }
 

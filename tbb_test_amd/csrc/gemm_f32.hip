@@ -827,17 +827,18 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
 // the registers the MFMAs read -- no LDS tile, no barrier in the loop (the operands of such small
 // problems sit in the L2).  The four partial blocks are added through the LDS in wavefront order
 // (deterministic), wavefront w finishing rows 8w .. 8w+7 of the block.
+// `tile` = index of the 32 x 32 block in row-major order, `z` = batch entry.
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM>
-__global__ __launch_bounds__(256) void gemm_f32_splitk(GemmArgs p) {
+__device__ __forceinline__ void splitk_block(const GemmArgs& p, int tile, int z) {
   __shared__ float part[4][16][64];
   __shared__ float cs_part[4][32];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hi = lane >> 5;
-  const int tile_m = blockIdx.x / p.tiles_n, tile_n = blockIdx.x - tile_m * p.tiles_n;
+  const int tile_m = tile / p.tiles_n, tile_n = tile - tile_m * p.tiles_n;
   const int m0 = tile_m * 32, n0 = tile_n * 32;
-  const float* __restrict__ A = p.A + (size_t)blockIdx.z * p.batchA;
-  const float* __restrict__ B = p.B + (size_t)blockIdx.z * p.batchB;
-  float* __restrict__ C = p.C + (size_t)blockIdx.z * p.batchC;
+  const float* __restrict__ A = p.A + (size_t)z * p.batchA;
+  const float* __restrict__ B = p.B + (size_t)z * p.batchB;
+  float* __restrict__ C = p.C + (size_t)z * p.batchC;
   const int kq = p.K / 4, k_begin = wave * kq, chunks = kq / 8;
   // lane (l32, hi) feeds MFMA step q of a chunk with k = chunk*8 + 4*hi + q
   const float* a_ptr = A_KMAJOR ? A + (size_t)(m0 + l32) * p.lda + k_begin + 4 * hi
@@ -893,7 +894,7 @@ __global__ __launch_bounds__(256) void gemm_f32_splitk(GemmArgs p) {
   }
   __syncthreads();
   if (COLSUM && do_colsum && tid < 32)
-    p.colsum[(size_t)blockIdx.z * p.batchColsum + m0 + tid] =
+    p.colsum[(size_t)z * p.batchColsum + m0 + tid] =
         ((cs_part[0][tid] + cs_part[1][tid]) + cs_part[2][tid]) + cs_part[3][tid];
   const int col = n0 + l32;
   const float bias_v = (EPI == EPI_BIAS_RELU && p.bias) ? p.bias[col] : 0.0f;
@@ -909,6 +910,27 @@ __global__ __launch_bounds__(256) void gemm_f32_splitk(GemmArgs p) {
       if (!(p.mask[(size_t)row * p.ldmask + col] > 0.0f)) v = 0.0f;
     }
     C[(size_t)row * p.ldc + col] = v;
+  }
+}
+
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM>
+__global__ __launch_bounds__(256) void gemm_f32_splitk(GemmArgs p) {
+  splitk_block<A_KMAJOR, B_KMAJOR, EPI, COLSUM>(p, blockIdx.x, blockIdx.z);
+}
+
+// The two backward GEMMs of one layer in one launch: the weight gradient (all replicas, bias
+// gradient fused) and the input gradient read the same dZ and depend on nothing of each other.  For
+// problems this small a step is a chain of launches of a few microseconds each, and one launch less
+// per layer is worth more than anything inside the kernels.  Workgroups [0, wgrad_blocks) run the
+// weight gradient (tile fastest, then replica), the rest the input gradient.
+template <int EPI_D>
+__global__ __launch_bounds__(256) void gemm_f32_splitk_pair(GemmArgs pw, GemmArgs pd, int wgrad_blocks) {
+  const int b = blockIdx.x;
+  if (b < wgrad_blocks) {
+    const int per = pw.tiles_m * pw.tiles_n, z = b / per;
+    splitk_block<false, false, EPI_NONE, true>(pw, b - z * per, z);
+  } else {
+    splitk_block<true, false, EPI_D, false>(pd, b - wgrad_blocks, 0);
   }
 }
 
@@ -1145,6 +1167,41 @@ hipError_t sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const f
   hipError_t e = dispatch<false, false, EPI_NONE, true>(p, R, s, variant, &fused);
   if (e != hipSuccess || fused) return e;
   return colsum_f32(R, M, K, A, lda, colsum, stride_colsum, s);  // any-shape path: separate kernel
+}
+
+// Whether the automatic choice takes the split-K kernel for a GEMM of this shape (the same rule
+// as in dispatch(): whole 32 x 32 blocks, K a multiple of 32, fewer 64 x 64 tiles than CUs).
+static bool splitk_shape(int M, int N, int K, int batch) {
+  return M > 0 && N > 0 && K > 0 && M % 32 == 0 && N % 32 == 0 && K % 32 == 0 &&
+         (long long)(M / 64) * (N / 64) * batch < 192 && (long long)(M / 128) * (N / 128) * batch * 2 < 192;
+}
+
+bool sgemm_backward_pair_fits(int R, int rows, int nout, int nin) {
+  // weight gradient: M = nout, N = nin, K = rows / R per replica; input gradient: M = rows, N = nin, K = nout
+  return R > 0 && rows % R == 0 && splitk_shape(nout, nin, rows / R, R) && splitk_shape(rows, nin, nout, 1) &&
+         nout % 4 == 0 && nin % 4 == 0;
+}
+
+hipError_t sgemm_backward_pair(int R, int rows, int nout, int nin, const float* dZ, const float* A, const float* W,
+                               float* dW, long long strideW, float* db, long long stride_db, float* dA,
+                               const float* mask, hipStream_t s) {
+  if (!sgemm_backward_pair_fits(R, rows, nout, nin) || !aligned16(dZ) || !aligned16(A) || !aligned16(W) ||
+      !aligned16(dW) || !aligned16(dA) || strideW % 4 != 0 || (mask && !aligned16(mask)))
+    return hipErrorInvalidValue;
+  const int Kw = rows / R;
+  GemmArgs pw{};
+  pw.M = nout; pw.N = nin; pw.K = Kw; pw.A = dZ; pw.B = A; pw.C = dW; pw.lda = nout; pw.ldb = nin; pw.ldc = nin;
+  pw.batchA = (long long)Kw * nout; pw.batchB = (long long)Kw * nin; pw.batchC = strideW;
+  pw.colsum = db; pw.batchColsum = stride_db;
+  pw.tiles_m = nout / 32; pw.tiles_n = nin / 32;
+  GemmArgs pd{};
+  pd.M = rows; pd.N = nin; pd.K = nout; pd.A = dZ; pd.B = W; pd.C = dA; pd.lda = nout; pd.ldb = nin; pd.ldc = nin;
+  pd.mask = mask; pd.ldmask = nin;
+  pd.tiles_m = rows / 32; pd.tiles_n = nin / 32;
+  const int wgrad_blocks = pw.tiles_m * pw.tiles_n * R, dgrad_blocks = pd.tiles_m * pd.tiles_n;
+  if (mask) launch_kernel(gemm_f32_splitk_pair<EPI_MASK>, dim3(wgrad_blocks + dgrad_blocks), dim3(256), 0, s, pw, pd, wgrad_blocks);
+  else launch_kernel(gemm_f32_splitk_pair<EPI_NONE>, dim3(wgrad_blocks + dgrad_blocks), dim3(256), 0, s, pw, pd, wgrad_blocks);
+  return hipGetLastError();
 }
 
 }  // namespace mi

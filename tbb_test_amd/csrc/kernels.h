@@ -78,6 +78,16 @@ hipError_t sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const f
                     float* C, int ldc, long long strideC, float* colsum, long long stride_colsum,
                     hipStream_t s, int variant);
 
+// Both backward GEMMs of one dense fp32 layer in one launch, for problems so small that a step is
+// bound by the number of launches (the shapes the automatic choice gives to the split-K kernel):
+//   dW_r[nout x nin] = dZ_r^T A_r, db_r = colsum dZ_r (r < R, rows / R rows each), dA[rows x nin] = dZ W (masked)
+// with dense operands dZ [rows x nout], A [rows x nin], W [nout x nin], mask [rows x nin] or null.
+// Same arithmetic, bit for bit, as sgemm_tn + sgemm_nn on those shapes.
+bool sgemm_backward_pair_fits(int R, int rows, int nout, int nin);
+hipError_t sgemm_backward_pair(int R, int rows, int nout, int nin, const float* dZ, const float* A, const float* W,
+                               float* dW, long long strideW, float* db, long long stride_db, float* dA,
+                               const float* mask, hipStream_t s);
+
 // gemv_f32.hip: the same three operations for layers whose output width is at most SKINNY_MAX
 // (N of the forward GEMM, M of the weight gradient, K of the input gradient), as matrix-vector
 // passes at memory speed.  Any alignment; the automatic choice of sgemm_* takes them.

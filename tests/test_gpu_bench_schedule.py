@@ -59,7 +59,8 @@ def test_config_2_benchmarked_schedule_full_size():
     h, X, Ws, dY = build(nf, B, R, seed=1, flags=BENCH_FLAGS)
     bench_loop(h, 4)            # step 1 eager, steps 2-4 replay the graph
     sched = h.schedule()
-    assert sched == {"dual_streams": True, "per_layer_update": True, "graph": True, "fused_transposes": 0}
+    assert sched == {"dual_streams": True, "per_layer_update": True, "graph": True, "fused_transposes": 0,
+                     "paired_backward": False}
 
     bs = [np.zeros(n, np.float32) for n in nf[1:]]
     ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR)
@@ -82,7 +83,8 @@ def test_config_2_benchmarked_schedule_full_size():
     # and bit for bit what the serial eager schedule computes (one stream, one update launch)
     hs, *_ = build(nf, B, R, seed=1, flags=capi.FLAG_NO_GRAPH | capi.FLAG_SERIAL_BACKWARD)
     bench_loop(hs, 1)
-    assert hs.schedule() == {"dual_streams": False, "per_layer_update": False, "graph": False, "fused_transposes": 0}
+    assert hs.schedule() == {"dual_streams": False, "per_layer_update": False, "graph": False, "fused_transposes": 0,
+                             "paired_backward": False}
     assert np.array_equal(bits(h.dx()), bits(hs.dx()))
     for l in range(L):
         assert np.array_equal(bits(h.weight(l)), bits(hs.weight(l))), f"W {l}"

@@ -146,9 +146,10 @@ def test_loss_without_labels_is_an_error():
     h.close()
 
 
+@pytest.mark.parametrize("nf", [[128, 256, 128, 64], [128, 200, 128, 64]], ids=["small", "ragged"])
 @pytest.mark.parametrize("flags", [0, capi.FLAG_PER_LAYER_UPDATE, capi.FLAG_SERIAL_BACKWARD])
-def test_trace_step_writes_reference_style_timeline(tmp_path, flags):
-    nf, B, R = [128, 256, 128, 64], 64, 2
+def test_trace_step_writes_reference_style_timeline(tmp_path, flags, nf):
+    B, R = 64, 2
     L = len(nf) - 1
     h, _ = build(nf, B, R, seed=9, flags=flags)
     h2, _ = build(nf, B, R, seed=9, flags=flags | capi.FLAG_NO_GRAPH)
@@ -161,9 +162,14 @@ def test_trace_step_writes_reference_style_timeline(tmp_path, flags):
     begins = [e for e in events if e["ph"] == "B"]
     assert len(events) == 2 * len(begins)
     names = sorted(e["name"] for e in begins)
-    expect = [f"FC_{l}_0" for l in range(L)] + [f"FCWgtGradient_{l}_0" for l in range(L)] + \
-             [f"FCBwdGradient_{l}_0" for l in range(L)] + ["L2Loss_0"]
-    if flags & capi.FLAG_PER_LAYER_UPDATE:
+    paired = h.schedule()["paired_backward"]
+    assert paired == (nf == [128, 256, 128, 64])   # the small model runs the fewest-launches schedule
+    if paired:
+        expect = [f"FC_{l}_0" for l in range(L)] + [f"FCWgtGradient+FCBwdGradient_{l}_0" for l in range(L)] + ["L2Loss_0"]
+    else:
+        expect = [f"FC_{l}_0" for l in range(L)] + [f"FCWgtGradient_{l}_0" for l in range(L)] + \
+                 [f"FCBwdGradient_{l}_0" for l in range(L)] + ["L2Loss_0"]
+    if flags & capi.FLAG_PER_LAYER_UPDATE and not paired:
         expect += [f"ReduceScatterAllGather_{l}_0" for l in range(L)]
     else:
         expect += ["ReduceScatterAllGather_all_0"]
@@ -175,12 +181,13 @@ def test_trace_step_writes_reference_style_timeline(tmp_path, flags):
         assert [e["ph"] for e in mine] == ["B", "E"] * (len(mine) // 2)
         ts = [e["ts"] for e in mine]
         assert all(b >= a for a, b in zip(ts, ts[1:])), ts
-    if flags & capi.FLAG_SERIAL_BACKWARD and not flags & capi.FLAG_PER_LAYER_UPDATE:
+    if paired or (flags & capi.FLAG_SERIAL_BACKWARD and not flags & capi.FLAG_PER_LAYER_UPDATE):
         assert all(e["tid"] == 0 for e in events)
     elif not flags & capi.FLAG_SERIAL_BACKWARD:
         assert any(e["tid"] == 1 for e in events)
-    # forward precedes backward: FC_{L-1} ends before FCBwdGradient_{L-1} begins
+    # forward precedes backward: FC_{L-1} ends before the backward of layer L-1 begins
     order = {e["name"]: e["ts"] for e in begins}
-    assert order[f"FC_{L - 1}_0"] <= order[f"FCBwdGradient_{L - 1}_0"]
+    first_bwd = f"FCWgtGradient+FCBwdGradient_{L - 1}_0" if paired else f"FCBwdGradient_{L - 1}_0"
+    assert order[f"FC_{L - 1}_0"] <= order[first_bwd]
     h.close()
     h2.close()
