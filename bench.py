@@ -34,29 +34,48 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 CONFIGS = {
-    # name: (layers, width, batch per replica, replicas, dtype)
-    "C1": (3, 512, 256, 2, "f32"),
-    "C2": (8, 1024, 1024, 4, "f32"),
-    "C3": (4, 4096, 2048, 2, "f32"),
-    "C4": (20, 2048, 256, 8, "f32"),
-    "C5": (8, 8192, 4096, 4, "bf16"),
+    # name: (layer widths N_0 .. N_L, batch per replica, replicas, dtype)
+    "C1": ([512] * 4, 256, 2, "f32"),
+    "C2": ([1024] * 9, 1024, 4, "f32"),
+    "C3": ([4096] * 5, 2048, 2, "f32"),
+    "C4": ([2048] * 21, 256, 8, "f32"),
+    "C5": ([8192] * 9, 4096, 4, "bf16"),
+    # the reference's own default model (mlp_bench_common.h:26), four sockets of 1024 rows
+    "ref": ([1024] * 7 + [1], 1024, 4, "f32"),
 }
 PEAK_TFLOPS = {"f32": 157.3, "bf16": 2516.6}  # MI355X dense MFMA peaks
 PEAK_HBM_GBPS = 8000.0
 METRIC = "MLP fwd+bwd+reduce step ms & TFLOP/s on 1 MI355X; grad-reduce GB/s"
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark
-# (FETCH_SIZE scaled by 1.9986, WRITE_SIZE by 1.0, the factors a plain 33.6 MB device copy gives;
-# the runs are summarised under profiles/).  GEMM: mean over the forward, weight-gradient and
-# input-gradient launches.  None = not measured for that configuration.
-MEASURED_TRAFFIC_BYTES = {
-    "C2": {"gemm": (50.4e6 + 16.8e6 + 50.4e6 + 16.8e6 + 67.2e6 + 16.8e6) / 3, "reduce": 167.8e6 + 33.6e6},
-    # configs 3-5: mean over the GEMM launches of a step (forward, weight gradient, input gradient
-    # with and without mask, weighted by their counts)
-    "C3": {"gemm": 911.7e6, "reduce": 805.5e6 + 268.5e6},
-    "C4": {"gemm": 189.3e6, "reduce": 3021.4e6 + 335.7e6},
-    "C5": {"gemm": 4010.5e6, "reduce": 10738.7e6 + 3221.6e6},
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic_pmc.json")
+KERNEL_SOURCES = os.path.join(ROOT, "tbb_test_amd", "csrc")
+
+
+def kernel_source_hash():
+    """sha256 over the kernel sources: the measured traffic figures belong to one state of them."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(KERNEL_SOURCES)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            h.update(open(os.path.join(KERNEL_SOURCES, name), "rb").read())
+    return h.hexdigest()
+
+
+def measured_traffic(config):
+    """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
+    scaled by what the same counter reads for the plain device copy of the weight restore), as
+    recorded in profiles/traffic_pmc.json together with the hash of the kernel sources they were
+    measured on.  Returns ({"gemm": bytes, "reduce": bytes}, note); figures are None when nothing
+    was recorded for the configuration or when the kernels have changed since."""
+    try:
+        data = json.load(open(TRAFFIC_FILE))
+    except (OSError, ValueError):
+        return {}, "no traffic file"
+    if data.get("source_hash") != kernel_source_hash():
+        return {}, "kernel sources changed since the counters were read (profiles/traffic_pmc.json is stale)"
+    return data.get("configs", {}).get(config, {}), data.get("how", "")
 
 
 def cpu_baseline(nf, B, R, lr, budget_s):
@@ -91,8 +110,8 @@ def main():
 
     from tbb_test_amd import capi, hostlib
 
-    layers, width, B, R, dtype = CONFIGS[args.config]
-    nf = [width] * (layers + 1)
+    nf, B, R, dtype = CONFIGS[args.config]
+    layers = len(nf) - 1
     info = capi.device_info()
 
     X, Ws, dY = hostlib.init_problem(nf, B, R, args.seed)
@@ -137,6 +156,7 @@ def main():
     ms, cnt = h.timings()
     h.enable_timing(False)
     finite = all(bool(np.isfinite(h.weight(l)).all()) for l in range(layers))
+    sched = h.schedule()     # what the timed loop actually ran (the library also looks at the shapes)
     h.close()
 
     # What the matrix cores sustain right now with no memory traffic at all (register-resident
@@ -154,10 +174,16 @@ def main():
                         "after the steps above (mi_probe_mfma_rate)"}
 
     rows = R * B
-    flop_per_gemm = 2.0 * rows * width * width          # every GEMM launch of a square model
-    gemm_flop_step = 3 * layers * flop_per_gemm
-    gemm_ms = float(ms[0:3].sum())
-    gemm_launches = int(cnt[0:3].sum())
+    # FLOP of the forward / weight-gradient / input-gradient GEMM of layer l: 2 * rows * N_l * N_{l+1}.
+    # The roofline object prices the dominant kernel: the GEMM launches of the widest layers (all of
+    # them in the square benchmark configurations; the 1024 -> 1 layer of `ref` runs on the
+    # matrix-vector kernels and is left out of the MFMA figure).
+    layer_flop = [2.0 * rows * nf[l] * nf[l + 1] for l in range(layers)]
+    gemm_flop_step = 3 * sum(layer_flop)
+    flop_per_gemm = max(layer_flop)
+    wide = [l for l in range(layers) if layer_flop[l] == flop_per_gemm]
+    gemm_ms = float(ms[0:3][:, wide].sum())
+    gemm_launches = int(cnt[0:3][:, wide].sum())
     gemm_avg_ms = gemm_ms / gemm_launches
     gemm_tflops = flop_per_gemm / (gemm_avg_ms * 1e-3) / 1e12
     per_phase = {capi.BREAKDOWN_NAMES[i]: float(ms[i].sum() / args.steps) for i in range(4)}
@@ -167,10 +193,15 @@ def main():
     # the event-timed pass always runs the update as one launch over all layers
     upd_bytes = (R + 2) * 4.0 * params
     if dtype == "bf16":
-        upd_bytes += 2.0 * params
+        upd_bytes += 4.0 * params   # the bf16 copy and the transposed bf16 copy of the weights
     upd_gbps = upd_bytes / (upd_ms * 1e-3) / 1e9
 
     peak = PEAK_TFLOPS[dtype]
+    traffic, traffic_note = measured_traffic(args.config)
+    schedule = ("weight and input gradient of a layer in one launch, one stream" if sched["paired_backward"]
+                else "weight-gradient GEMMs on a second stream" if sched["dual_streams"] else "backward pass on one stream")
+    schedule += ", per-layer update on the second stream" if sched["per_layer_update"] else ", one update launch"
+    schedule += ", graph replay" if sched["graph"] else ", eager launches"
     out = {
         "metric": METRIC,
         "value": round(gemm_flop_step / (ms_per_step * 1e-3) / 1e12, 3),
@@ -184,26 +215,27 @@ def main():
         "vs_baseline": None,
         "dtype": dtype,
         "data": "synthetic",
-        "config": {"workload": f"{args.config}: {layers} FC layers of width {width}, ReLU between layers, "
-                               f"batch {B} per replica x {R} replicas, lr {args.lr}, seed {args.seed}",
-                   "schedule": ("serial backward" if args.serial_backward or args.config in ("C3", "C5")
-                                else "weight-gradient GEMMs on a second stream")
-                               + (", one update launch" if args.flat_update else ", per-layer update on the second stream"),
-                   "device": info["name"], "num_cus": info["num_cus"]},
+        "config": {"workload": f"{args.config}: {layers} FC layers, widths "
+                               + (f"{nf[0]} throughout" if len(set(nf)) == 1 else " ".join(str(v) for v in nf))
+                               + f", ReLU between layers, batch {B} per replica x {R} replicas, lr {args.lr}, seed {args.seed}",
+                   "schedule": schedule, "device": info["name"], "num_cus": info["num_cus"]},
         "gemm_flop_per_step": gemm_flop_step,
         "phase_ms_per_step": {k: round(v, 4) for k, v in per_phase.items()},
         "gemm_tflops": round(gemm_tflops, 2),
         "reduce_gbps": round(upd_gbps, 1),
         "weights_finite": finite,
-        "roofline": {"kernel": "gemm_f32_dma (nt, nn, tn)" if dtype == "f32" else "gemm_bf16_dma",
+        "roofline": {"kernel": "gemm_f32_dma (nt, nn, tn)" if dtype == "f32" else
+                               "gemm_bf16_dma (spans of the weight gradient include its row-sum kernel and, for "
+                               "operands no GEMM epilogue wrote transposed, the transpose launches)",
                      "bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(gemm_tflops / peak, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get("gemm"),
+                     "traffic": traffic.get("gemm"), "traffic_note": traffic_note,
                      "flop_per_launch": flop_per_gemm, "avg_launch_us": round(gemm_avg_ms * 1e3, 2),
                      "launches": gemm_launches, "mfma_only_rate": mfma_only},
-        "roofline_reduce": {"kernel": "reduce_sgd_vec4", "bound": "hbm", "achieved": round(upd_gbps, 1),
+        "roofline_reduce": {"kernel": "reduce_sgd_vec4" if dtype == "f32" else "reduce_sgd_tile (one launch per layer)",
+                            "bound": "hbm", "achieved": round(upd_gbps, 1),
                             "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(upd_gbps / PEAK_HBM_GBPS, 4),
-                            "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get("reduce"),
+                            "traffic": traffic.get("reduce"),
                             "bytes_per_launch": upd_bytes, "avg_launch_us": round(upd_ms * 1e3, 2)},
     }
     if args.cpu_seconds > 0:

@@ -269,8 +269,8 @@ int mi_mlp_restore_weights(mi_mlp* h);
  * [N_l x N_{l+1}]), widened to fp32.  Both are rewritten by every update.  Synchronous. */
 int mi_mlp_get_weight_shadow(mi_mlp* h, int l, int transposed, float* dst, int ld);
 
-/* What the last mi_mlp_step / mi_mlp_trace_step actually did (the scheduling flags are requests;
- * the library also looks at the shapes and at whether per-kernel timing is on):
+/* What the last mi_mlp_step / mi_mlp_trace_step outside per-kernel timing actually did (the
+ * scheduling flags are requests; the library also looks at the shapes):
  *   info[0]  1 = backward pass on two streams, 0 = on one
  *   info[1]  1 = one update launch per layer on the second stream, 0 = one launch at the end
  *   info[2]  1 = steps replay a captured HIP graph

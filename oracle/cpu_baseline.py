@@ -131,6 +131,23 @@ def run(nf, B, R, lr, budget_s):
                   f"{R} replicas x {T} threads = {R * T} OpenMP threads on {cores} host cores, restatement of "
                   "mlp_omp (oracle/mlp_omp_port.c)",
     }
+    # The same figures in the units and wording of the reference's report_timing()
+    # (mlp_bench_common.cc:92-149): GF/s per core for the GEMM phases (mlp_omp.cc:492,584,675 count
+    # 2 m n k per phase), GB/s per socket for the update with the reference's byte model
+    # 2 (sockets - 1) * 4 * sum rows * cols (reduce-scatter + all-gather, mlp_omp.cc:163,288).  The
+    # port keeps per-phase totals only, so the per-layer lines and the imbalance column are not given.
+    nthreads = R * T
+    phase_flop = 2.0 * R * B * sum(nf[l] * nf[l + 1] for l in range(L))
+    ring_bytes = 2.0 * (R - 1) * 4.0 * sum(nf[l] * nf[l + 1] for l in range(L))
+
+    def rate(amount, t_ms, per):
+        return amount / (t_ms * 1e-3) / per / 1e9 if t_ms > 0 else 0.0
+    out["report_timing"] = (
+        f"total fwd {t[0]:g} ms/iter ({rate(phase_flop, t[0], nthreads):g} GF/s/core), "
+        f"wgt_grad {t[1]:g} ms/iter ({rate(phase_flop, t[1], nthreads):g} GF/s/core), "
+        f"bwd {t[2]:g} ms/iter ({rate(phase_flop, t[2], nthreads):g} GF/s/core), "
+        f"wgt_update {t[3]:g} ms/iter ({rate(ring_bytes, t[3], R):g} GB/s/socket); "
+        f"wall clock time {ms:g} ms/iter")
     dag_iters = int(max(1, min(100, (budget_s / 3 - est) / est)))
     _, _, td = run_port(nf, B, R, T, lr, X, dY, W_flat, 1, dag_iters, scheduler="dag")
     out["task_graph"] = {

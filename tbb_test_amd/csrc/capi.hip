@@ -553,9 +553,11 @@ int enqueue_step(mi_mlp* h, float lr) {
   // 3, 1024 tiles: 11.32 ms with one backward stream, 11.47 ms with two; config 5: 45.9 / 47.1 ms).
   const bool crowded = (long long)(h->MB / 128) * (long long)(h->maxw() / 128) >= 1024;
   const bool dual = !(h->flags & MI_FLAG_SERIAL_BACKWARD) && !h->timing && !crowded && !paired;
-  h->last_dual = dual;
-  h->last_per_layer = per_layer;
-  h->last_paired = paired;
+  if (!h->timing) {  // the per-kernel timing pass is not the schedule mi_mlp_get_schedule reports
+    h->last_dual = dual;
+    h->last_per_layer = per_layer;
+    h->last_paired = paired;
+  }
   hipStream_t s2 = dual ? h->stream2 : s;
   if (dual) {  // fork: dZ_{L-1} and all activations are ready
     MI_HIP(hipEventRecord(h->ev_fork, s));

@@ -217,8 +217,9 @@ int main(int argc, char** argv) {
     // bytes the update has to move: R gradient copies in, W in, W out
     const double layer_params = (double)model.nfeatures[l] * model.nfeatures[l + 1] + model.nfeatures[l + 1];
     const double bytes = (R + 2) * 4.0 * layer_params * NITER;
-    if (flags & MI_FLAG_PER_LAYER_UPDATE) sum_flops[l][WGT_UPDATE] = bytes;
-    else sum_flops[0][WGT_UPDATE] += bytes;  // one launch over all layers, booked on layer 0
+    // the per-kernel timing pass always runs the update as one launch over all layers (overlapping
+    // launches cannot be timed one by one), whatever schedule the timed loop used: layer 0 carries it
+    sum_flops[0][WGT_UPDATE] += bytes;
   }
 
   /////////////////////////////////////////////////////////////////////////////
