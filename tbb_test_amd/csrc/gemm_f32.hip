@@ -63,6 +63,8 @@ struct GemmArgs {
   // tile rasterisation (flat grid of tiles_m * tiles_n * batch workgroups)
   int tiles_m, tiles_n, batch;
   int raster, per_xcd, total_shift, tiles_n_shift;  // see tile_of_block / set_raster
+  // CHAIN instances of gemm_f32_dma: number of batch entries a workgroup walks through
+  int chain;
 };
 
 // Maps the flat workgroup index to a batch entry and a C tile.  Workgroups are handed to the 8
@@ -645,8 +647,23 @@ __device__ __forceinline__ void load_frag_swz(float (&frag)[TB][4], const float*
   }
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM, int STAGES>
+// CHAIN = true (weight gradient with a short K per replica): the replicas of one launch are
+// consecutive ranges of K rows of both operands (batchA = K * lda, batchB = K * ldb), so a
+// workgroup that keeps its (m, n) tile and walks through all p.chain replicas sees one long K loop
+// whose ring of tile loads never drains; every p.K / BK steps it stores the accumulators as that
+// replica's C tile (and the column sums as its bias gradient), clears them and goes on.  Prologue
+// and epilogue are paid once per workgroup instead of once per replica, and the stores of a replica
+// drain under the next replica's MFMAs: the wait in front of the next ring barrier lets them stay
+// in flight (vmcnt retires in order, and the tile that barrier needs was requested before them).
+// Measured on 20 layers of 2048 x 2048 with 8 replicas of 256 rows: 129 us per launch against
+// 139 us for one workgroup per (replica, tile) -- but the whole step gets slower (8.1-8.5 ms against
+// 7.9 ms): the short workgroups of the plain kernel fill the prologue and epilogue gaps of the
+// input-gradient chain on the other stream, these long-lived ones only compete with it.  Hence
+// not part of the automatic choice; mi_set_gemm_variant(2, 35) selects it.
+template <int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM, int STAGES,
+          bool CHAIN = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
+  static_assert(!CHAIN || (!A_KMAJOR && !B_KMAJOR && EPI == EPI_NONE), "chained replicas: weight gradient only");
   constexpr int NW = WM * WN, NT = NW * 64;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -676,6 +693,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
   tile_of_block(p, tile_m, tile_n, bz);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   float* __restrict__ C = p.C + (size_t)bz * p.batchC;
+  float* __restrict__ colsum_out = COLSUM && p.colsum ? p.colsum + (size_t)bz * p.batchColsum + m0 : nullptr;
 
   // Global source of the load instructions: a wave-uniform base pointer per operand (the tile's
   // first element for the current K step, advanced with scalar adds) plus a constant 32-bit byte
@@ -745,7 +763,13 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
   const bool do_colsum = COLSUM && p.colsum != nullptr && tile_n == 0;
   float csum = 0.0f;
 
-  const int nk = p.K / BK;
+  const int steps_per_entry = p.K / BK;                       // CHAIN: K steps per replica
+  const int nk = CHAIN ? steps_per_entry * p.chain : steps_per_entry;
+  int steps_left = steps_per_entry;                           // CHAIN: steps until the accumulators are stored
+  bool stores_in_flight = false;                              // CHAIN: the previous step ended with a store burst
+  // one float per thread behind the ring: partial column sums of a replica (CHAIN; the ring itself is never idle)
+  float* cs_smem = smem + STAGES * (A_FLOATS + B_FLOATS);
+  constexpr int TILE_STORES = TM * TN * 16 / ((!B_KMAJOR && (TN == 2 || TN == 4)) ? TN : 1);  // store instructions of write_tile per wave
 #pragma unroll
   for (int st = 0; st < STAGES - 1; ++st)
     if (st < nk) issue(st);
@@ -781,8 +805,15 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
         // empty MFMA pipe (measured: every such step 12 % longer).
         __builtin_amdgcn_sched_barrier(0);
         // tiles t+1 .. t+STAGES-2 are in flight; tile t+1 must have landed
-        if (steady || t + STAGES - 2 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_only((STAGES - 3) * INSTR));
-        else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+        if (CHAIN && stores_in_flight) {
+          // the stores of the replica that ended with the previous step are younger than every load
+          // that has to be complete here: they may stay outstanding
+          if (steady || t + STAGES - 2 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_only((STAGES - 3) * INSTR + TILE_STORES));
+          else __builtin_amdgcn_s_waitcnt(vmcnt_only(TILE_STORES));
+        } else {
+          if (steady || t + STAGES - 2 < nk) __builtin_amdgcn_s_waitcnt(vmcnt_only((STAGES - 3) * INSTR));
+          else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+        }
         ring_barrier();
         if (steady || t + STAGES - 1 < nk) issue(fill);
       }
@@ -790,6 +821,34 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
         const float* col = As(cur) + (tid / BM) * CS_ROWS * BM + (tid % BM);
 #pragma unroll
         for (int k = 0; k < CS_ROWS; ++k) csum += col[k * BM];
+      }
+    }
+    if constexpr (CHAIN) {
+      stores_in_flight = false;
+      if (--steps_left == 0 && t + 1 < nk) {  // a replica is complete (the last one leaves through the epilogue below)
+        steps_left = steps_per_entry;
+        if (COLSUM && do_colsum) {  // uniform over the workgroup
+          cs_smem[tid] = csum;
+          csum = 0.0f;
+          lds_barrier();
+          if (tid < BM) {
+            float total = cs_smem[tid];
+#pragma unroll
+            for (int sl = 1; sl < CS_SLICES; ++sl) total += cs_smem[sl * BM + tid];
+            colsum_out[tid] = total;
+          }
+          colsum_out += p.batchColsum;
+          // cs_smem is written again one replica later at the earliest, i.e. behind a ring barrier
+        }
+        write_tile<TM, TN, A_KMAJOR, B_KMAJOR, EPI, false>(p, C, acc, m0 + wm0, n0 + wn0, lane);
+        C += p.batchC;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+        stores_in_flight = true;
       }
     }
   };
@@ -812,7 +871,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
       float total = smem[tid];
 #pragma unroll
       for (int sl = 1; sl < CS_SLICES; ++sl) total += smem[sl * BM + tid];
-      p.colsum[(size_t)bz * p.batchColsum + m0 + tid] = total;
+      colsum_out[tid] = total;
     }
   }
   write_tile<TM, TN, A_KMAJOR, B_KMAJOR, EPI, false>(p, C, acc, m0 + wm0, n0 + wn0, lane);
@@ -1021,13 +1080,18 @@ static hipError_t launch_mfma(GemmArgs& p, int batch, hipStream_t s) {
 // on its own; co-resident ones only interfere, and with several rounds of workgroups they make the
 // hardware's hand-out of workgroups to CUs uneven (measured on 1024 tiles: launches of 910 us and
 // of 1120 us at random with three 48 KB workgroups per CU, 910 us always with one).
-template <int BM, int BN, int BK, int WM, int WN, bool AK, bool BKM, int EPI, bool COLSUM, int STAGES>
+template <int BM, int BN, int BK, int WM, int WN, bool AK, bool BKM, int EPI, bool COLSUM, int STAGES, bool CHAIN = false>
 static hipError_t launch_dma(GemmArgs& p, int batch, hipStream_t s, bool exclusive = false) {
-  constexpr size_t lds_bytes = STAGES * (size_t)(BM + BN) * BK * sizeof(float);
+  // CHAIN: one float per thread behind the ring for the column-sum partials of a replica
+  constexpr size_t lds_bytes = STAGES * (size_t)(BM + BN) * BK * sizeof(float) + (CHAIN ? WM * WN * 64 * sizeof(float) : 0);
   static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB of LDS");
   constexpr size_t kExclusiveBytes = 84 * 1024;
   const size_t request = exclusive && lds_bytes < kExclusiveBytes ? kExclusiveBytes : lds_bytes;
-  auto kern = gemm_f32_dma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES>;
+  auto kern = gemm_f32_dma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES, CHAIN>;
+  if (CHAIN) {  // the workgroup walks the batch itself: the grid covers one entry's tiles
+    p.chain = batch;
+    batch = 1;
+  }
   static LdsOptIn opt_in;
   if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), request); e != hipSuccess) return e;
   p.tiles_m = p.M / BM;
@@ -1122,6 +1186,14 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
     case 31: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 33: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 34: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s, true); } break;
+    case 35:
+      if constexpr (!AK && !BKM && EPI == EPI_NONE) {
+        if (fits(128, 128, 16) && batch >= 1 && p.batchA == (long long)p.K * p.lda && p.batchB == (long long)p.K * p.ldb) {
+          if (fused_colsum) *fused_colsum = COLSUM;
+          return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3, true>(p, batch, s);
+        }
+      }
+      break;
     case 50: if (fits(32, 32, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_splitk<AK, BKM, EPI, COLSUM>(p, batch, s); } break;
     default: break;
   }

@@ -87,6 +87,8 @@ GEMM_SHAPES = [
     (1024, 384, 64), (4096, 3072, 32),
     # K loops of the direct-load kernels: a single step, and the longest conditional tail of a ring of four
     (128, 128, 16), (128, 128, 320),
+    # the short-K weight gradient with chained replicas at its own size (2048 x 2048 outputs, K = 256 per replica)
+    (2048, 2048, 256),
     (1, 1, 1), (5, 3, 7), (100, 130, 50), (129, 127, 33), (257, 64, 1000), (64, 1, 64), (1, 300, 17),
     # ragged but 16-byte aligned storage: the guarded MFMA kernels
     (132, 260, 100), (1000, 520, 200), (36, 4, 64), (300, 128, 36), (128, 300, 4),
@@ -94,7 +96,7 @@ GEMM_SHAPES = [
     # 16): the matrix-vector kernels, at the shapes of the reference's default last layer 1024 -> 1
     (4096, 1, 1024), (1, 1024, 1024), (4096, 1024, 1), (333, 16, 130), (16, 333, 130), (130, 333, 16), (50, 7, 1030),
 ]
-VARIANTS = [0, 8, 9, 10, 11, 12, 15, 16, 17, 21, 22, 30, 31, 33, 34, 50]
+VARIANTS = [0, 8, 9, 10, 11, 12, 15, 16, 17, 21, 22, 30, 31, 33, 34, 35, 50]   # 35: weight gradient, one workgroup walks all replicas
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
