@@ -85,6 +85,10 @@ struct mi_mlp {
   std::vector<uint16_t*> dzT;
   std::vector<char> actsT_fused;  // [L]
   std::vector<char> dzT_fused;  // [ndz]
+  // bf16 only: the per-replica transposed copy of the uploaded dY, made once by mi_mlp_set_dy (the
+  // weight gradient of the last layer reads it every step; the rotation buffers get overwritten)
+  uint16_t* dyT = nullptr;
+  bool dyT_valid = false;
   std::vector<void*> acts;    // L+1 buffers [MB x nf[l]], fp32 or bf16
   void* dy = nullptr;         // upstream gradient [MB x nf[L]]
   std::vector<void*> dz;      // [ndz] buffers of [MB x max width]
@@ -256,11 +260,14 @@ int op_wgrad(mi_mlp* h, int l, hipStream_t s, bool with_bias) {
     // possible, else from a transpose here)
     uint16_t* dzt = h->dzT[l % h->ndz];
     e = hipSuccess;
+    // the uploaded dY is the last layer's dZ as it stands (no ReLU after the last layer, no loss front-end)
+    const bool dy_cached = l == h->L - 1 && h->dyT_valid && !h->use_loss && !(h->flags & MI_FLAG_RELU_LAST);
+    if (dy_cached) dzt = h->dyT;
     if (!h->actsT_fused[l])
       e = mi::transpose_bf16(h->R, B, nin, (const uint16_t*)h->acts[l], nin, (long long)B * nin, h->actsT[l], B,
                              (long long)nin * B, s);
     const bool dz_fused = l < h->L - 1 && h->dzT_fused[l % h->ndz];  // the last layer's dZ is the given or derived dY
-    if (e == hipSuccess && !dz_fused)
+    if (e == hipSuccess && !dz_fused && !dy_cached)
       e = mi::transpose_bf16(h->R, B, nout, (const uint16_t*)dz_of_layer(h, l), nout, (long long)B * nout, dzt, B,
                              (long long)nout * B, s);
     if (e == hipSuccess)
@@ -943,6 +950,7 @@ int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_repli
     h->dzT.assign(h->ndz, nullptr);
     h->dzT_fused.assign(h->ndz, 0);
     for (int i = 0; i < h->ndz; ++i) alloc((void**)&h->dzT[i], (size_t)h->MB * h->maxw() * 2);
+    alloc((void**)&h->dyT, (size_t)h->MB * h->nf[L] * 2);
     h->actsT_fused.assign(L, 0);
     size_t wmax = 0;
     for (int l = 0; l < L; ++l) wmax = std::max(wmax, (size_t)h->nf[l] * h->nf[l + 1]);
@@ -1006,6 +1014,7 @@ int mi_mlp_destroy(mi_mlp* h) {
   (void)hipFree(h->params16T_saved);
   for (auto a : h->actsT) (void)hipFree(a);
   for (auto a : h->dzT) (void)hipFree(a);
+  (void)hipFree(h->dyT);
   for (void* a : h->acts) (void)hipFree(a);
   (void)hipFree(h->dy);
   for (void* a : h->dz) (void)hipFree(a);
@@ -1047,9 +1056,24 @@ int mi_mlp_set_weights(mi_mlp* h, int l, const float* W, int ld, const float* b)
   return MI_OK;
 }
 
+// bf16 models: the K-contiguous per-replica copy a weight-gradient GEMM reads, made once at upload
+// for the two operands that no GEMM of the step produces (the input X and a given dY)
+static int transposed_copy(mi_mlp* h, const void* src, int cols, uint16_t* dst) {
+  hipError_t e = mi::transpose_bf16(h->R, h->B, cols, (const uint16_t*)src, cols, (long long)h->B * cols, dst, h->B,
+                                    (long long)cols * h->B, h->stream);
+  if (e != hipSuccess) return hip_fail(e, "transpose launch");
+  MI_HIP(hipStreamSynchronize(h->stream));
+  return MI_OK;
+}
+
 int mi_mlp_set_input(mi_mlp* h, const float* X, int ld) {
   if (int rc = check_handle(h)) return rc;
-  return upload_matrix(h, h->acts[0], X, h->MB, h->nf[0], ld, h->dtype == MI_BF16);
+  if (int rc = upload_matrix(h, h->acts[0], X, h->MB, h->nf[0], ld, h->dtype == MI_BF16)) return rc;
+  if (h->dtype == MI_BF16) {
+    if (int rc = transposed_copy(h, h->acts[0], h->nf[0], h->actsT[0])) return rc;
+    h->actsT_fused[0] = 1;  // nothing in a step writes X, so the copy stays valid
+  }
+  return MI_OK;
 }
 
 int mi_mlp_set_dy(mi_mlp* h, const float* dY, int ld) {
@@ -1060,7 +1084,12 @@ int mi_mlp_set_dy(mi_mlp* h, const float* dY, int ld) {
     h->use_loss = false;
     drop_graph(h);
   }
-  return upload_matrix(h, h->dy, dY, h->MB, h->nf[h->L], ld, h->dtype == MI_BF16);
+  if (int rc = upload_matrix(h, h->dy, dY, h->MB, h->nf[h->L], ld, h->dtype == MI_BF16)) return rc;
+  if (h->dtype == MI_BF16) {
+    if (int rc = transposed_copy(h, h->dy, h->nf[h->L], h->dyT)) return rc;
+    h->dyT_valid = true;
+  }
+  return MI_OK;
 }
 
 int mi_mlp_set_labels(mi_mlp* h, const float* Y, int ld) {
