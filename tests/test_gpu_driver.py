@@ -27,6 +27,38 @@ def test_driver_runs_config_and_prints_report_and_checksum():
     assert "nan" not in text.lower()
 
 
+def test_report_timing_figures_are_consistent():
+    """The per-layer lines of report_timing (format of mlp_bench_common.cc:92-149): the rate printed
+    for a phase is the phase's FLOP (2 * rows * N_l * N_{l+1}, mlp_omp.cc:492,584,675) over the
+    printed time, the total line adds the layers up, and the update moves (R + 2) * 4 bytes per
+    parameter."""
+    text = run("4", "--config", "C2", "--warmup", "2", "--iters", "5")
+    rows, width, L, R = 4 * 1024, 1024, 8, 4
+    flop = 2.0 * rows * width * width
+    pat = re.compile(r"\[layer (\d+)\] fwd ([0-9.e+-]+) ms/iter \(([0-9.e+-]+) TF/s\), wgt_grad ([0-9.e+-]+) ms/iter "
+                     r"\(([0-9.e+-]+) TF/s\), bwd ([0-9.e+-]+) ms/iter \(([0-9.e+-]+) TF/s\), wgt_update ([0-9.e+-]+) ms/iter "
+                     r"\(([0-9.e+-]+) GB/s\)")
+    lines = pat.findall(text)
+    assert len(lines) == L, text
+    sums = [0.0, 0.0, 0.0]
+    for l, *vals in lines:
+        vals = [float(v) for v in vals]
+        for k in range(3):
+            ms, tf = vals[2 * k], vals[2 * k + 1]
+            assert ms > 0 and abs(tf - flop / (ms * 1e-3) / 1e12) <= 1e-3 * tf, (l, k, ms, tf)
+            assert 20 < tf < 157.3          # an fp32 GEMM rate below the MFMA peak
+            sums[k] += ms
+    upd_ms, upd_gbs = float(lines[0][7]), float(lines[0][8])   # the timed pass runs one update launch, booked on layer 0
+    params = L * (width * width + width)
+    assert abs(upd_gbs - (R + 2) * 4.0 * params / (upd_ms * 1e-3) / 1e9) <= 1e-3 * upd_gbs
+    assert all(float(line[7]) == 0 for line in lines[1:])
+    m = re.search(r"total fwd ([0-9.e+-]+) ms/iter \(([0-9.e+-]+) TF/s\), wgt_grad ([0-9.e+-]+) ms/iter", text)
+    assert m and abs(float(m.group(1)) - sums[0]) <= 1e-3 * sums[0]
+    assert abs(float(m.group(2)) - L * flop / (sums[0] * 1e-3) / 1e12) <= 1e-3 * float(m.group(2))
+    wall = float(re.search(r"wall clock time ([0-9.e+-]+) ms/iter", text).group(1))
+    assert 0.8 * sum(sums) < wall < 2.0 * sum(sums)
+
+
 def test_driver_is_deterministic_across_schedules():
     """Same seed, same checksum lines whether the step is replayed from a graph, launched kernel by
     kernel, or updates per layer on the second stream."""

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 import oracle
-from conftest import FP32_TOL, rel_err
+from conftest import FP32_TOL, close, rel_err
 from tbb_test_amd import capi
 
 pytestmark = pytest.mark.gpu
@@ -30,16 +30,17 @@ def bits_equal(a, b):
 
 
 def compare_step(h, ref, nf, R, tol=FP32_TOL, forward=True):
+    """Norm-wise and element-wise bound on everything a step produces."""
     L = len(nf) - 1
     for l in range(L + 1 if forward else 0):
-        assert rel_err(h.activation(l), ref.acts[l]) <= tol, f"activation {l}"
-    assert rel_err(h.dx(), ref.dX) <= tol, "dX"
+        assert close(h.activation(l), ref.acts[l], tol), f"activation {l}"
+    assert close(h.dx(), ref.dX, tol), "dX"
     for l in range(L):
         for r in range(R):
-            assert rel_err(h.wgrad_of(l, r), ref.dW[r][l]) <= tol, f"dW layer {l} replica {r}"
-            assert rel_err(h.bgrad_of(l, r), ref.db[r][l]) <= tol, f"db layer {l} replica {r}"
-        assert rel_err(h.weight(l), ref.W_new[l]) <= tol, f"updated W {l}"
-        assert rel_err(h.bias(l), ref.b_new[l]) <= tol, f"updated b {l}"
+            assert close(h.wgrad_of(l, r), ref.dW[r][l], tol), f"dW layer {l} replica {r}"
+            assert close(h.bgrad_of(l, r), ref.db[r][l], tol), f"db layer {l} replica {r}"
+        assert close(h.weight(l), ref.W_new[l], tol), f"updated W {l}"
+        assert close(h.bias(l), ref.b_new[l], tol), f"updated b {l}"
 
 
 CONFIGS = {
