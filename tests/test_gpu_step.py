@@ -157,3 +157,41 @@ def test_benchmark_config_2_full_size():
     ref_b = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR, given_acts=acts)
     compare_step(h, ref_b, nf, R, forward=False)
     h.close()
+
+
+def test_distinct_handles_on_distinct_threads():
+    """Two host threads, each with a handle of its own (different shapes, so different kernels and
+    LDS opt-ins), stepping at the same time: same bits as the same two models run one after the
+    other.  The binding releases the GIL inside every library call."""
+    import threading
+
+    models = [([512, 1024, 512], 256, 2, 21), ([256, 384, 128, 640], 128, 3, 22)]
+
+    def run(nf, B, R, seed, out, steps=4):
+        try:
+            h, _ = build(nf, B, R, seed=seed, flags=capi.FLAG_PER_LAYER_UPDATE)
+            for _ in range(steps):
+                h.step(1e-4)
+            h.sync()
+            out.append([h.weight(l) for l in range(len(nf) - 1)] + [h.dx()])
+            h.close()
+        except Exception as e:  # surfaces in the main thread
+            out.append(e)
+
+    serial = []
+    for nf, B, R, seed in models:
+        res = []
+        run(nf, B, R, seed, res)
+        serial.append(res[0])
+    for _ in range(3):
+        results = [[] for _ in models]
+        threads = [threading.Thread(target=run, args=(*m, results[i])) for i, m in enumerate(models)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=120)
+            assert not t.is_alive()
+        for want, got in zip(serial, results):
+            assert got and not isinstance(got[0], Exception), got
+            for a, b in zip(want, got[0]):
+                assert bits_equal(a, b)
