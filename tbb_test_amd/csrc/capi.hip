@@ -1321,12 +1321,12 @@ int mi_mlp_get_dx(mi_mlp* h, float* dst, int ld) {
 int mi_mlp_snapshot_weights(mi_mlp* h) {
   if (int rc = check_handle(h)) return rc;
   if (!h->params_saved) MI_HIP(hipMalloc((void**)&h->params_saved, h->stride * 4));
-  MI_HIP(hipMemcpyAsync(h->params_saved, h->params, h->stride * 4, hipMemcpyDeviceToDevice, h->stream));
+  MI_HIP(mi::device_copy(h->params_saved, h->params, h->stride * 4, h->stream));
   if (h->params16) {
     if (!h->params16_saved) MI_HIP(hipMalloc((void**)&h->params16_saved, h->stride * 2));
     if (!h->params16T_saved) MI_HIP(hipMalloc((void**)&h->params16T_saved, h->stride * 2));
-    MI_HIP(hipMemcpyAsync(h->params16_saved, h->params16, h->stride * 2, hipMemcpyDeviceToDevice, h->stream));
-    MI_HIP(hipMemcpyAsync(h->params16T_saved, h->params16T, h->stride * 2, hipMemcpyDeviceToDevice, h->stream));
+    MI_HIP(mi::device_copy(h->params16_saved, h->params16, h->stride * 2, h->stream));
+    MI_HIP(mi::device_copy(h->params16T_saved, h->params16T, h->stride * 2, h->stream));
   }
   return MI_OK;
 }
@@ -1334,10 +1334,10 @@ int mi_mlp_snapshot_weights(mi_mlp* h) {
 int mi_mlp_restore_weights(mi_mlp* h) {
   if (int rc = check_handle(h)) return rc;
   MI_REQUIRE(h->params_saved != nullptr, "no snapshot taken");
-  MI_HIP(hipMemcpyAsync(h->params, h->params_saved, h->stride * 4, hipMemcpyDeviceToDevice, h->stream));
+  MI_HIP(mi::device_copy(h->params, h->params_saved, h->stride * 4, h->stream));
   if (h->params16) {
-    MI_HIP(hipMemcpyAsync(h->params16, h->params16_saved, h->stride * 2, hipMemcpyDeviceToDevice, h->stream));
-    MI_HIP(hipMemcpyAsync(h->params16T, h->params16T_saved, h->stride * 2, hipMemcpyDeviceToDevice, h->stream));
+    MI_HIP(mi::device_copy(h->params16, h->params16_saved, h->stride * 2, h->stream));
+    MI_HIP(mi::device_copy(h->params16T, h->params16T_saved, h->stride * 2, h->stream));
   }
   return MI_OK;
 }

@@ -139,6 +139,9 @@ hipError_t transpose_bf16(int batch, int rows, int cols, const uint16_t* src, in
 hipError_t rowsum_bf16(int batch, int rows, int cols, const uint16_t* src, int ld, long long batch_src, float* out,
                        long long stride_out, hipStream_t s);
 
+// dst[0..bytes) = src[0..bytes) on the device (16-byte aligned: own kernel; else the runtime's copy)
+hipError_t device_copy(void* dst, const void* src, size_t bytes, hipStream_t s);
+
 hipError_t convert_f32_to_bf16(uint16_t* dst, const float* src, size_t n, hipStream_t s);
 hipError_t convert_bf16_to_f32(float* dst, const uint16_t* src, size_t n, hipStream_t s);
 
