@@ -100,7 +100,6 @@ struct mi_mlp {
   std::vector<hipEvent_t> ev_layer;  // per layer: input-gradient GEMM of layer l done (dZ_{l-1} ready, W_l free)
   std::vector<hipEvent_t> ev_wgrad;  // per layer: weight-gradient GEMM of layer l done (dZ_l free)
 
-  bool corun = false;  // set while enqueue_step issues an input-gradient GEMM next to a short-K weight gradient
 
   // loss front-end: when labels are set, every step derives dY from the forward output
   float* labels = nullptr;         // [MB x nf[L]] fp32
@@ -306,7 +305,7 @@ int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
   if (h->dtype == MI_F32) {
     e = mi::sgemm_nn(h->MB, h->nf[l], h->nf[l + 1], (const float*)dz_of_layer(h, l), h->nf[l + 1],
                      h->params + h->woff[l], h->nf[l], (float*)out, h->nf[l], (const float*)mask, h->nf[l], s,
-                     g_variant[1].load() ? g_variant[1].load() : (h->corun ? 100 : 0));
+                     g_variant[1]);
   } else {
     bool wrote = false;
     uint16_t* ct = (l > 0) ? h->dzT[(l - 1) % h->ndz] : nullptr;  // dZ_{l-1}^T for the weight gradient of layer l-1
@@ -570,23 +569,11 @@ int enqueue_step(mi_mlp* h, float lr) {
     MI_HIP(hipEventRecord(h->ev_fork, s));
     MI_HIP(hipStreamWaitEvent(s2, h->ev_fork, 0));
   }
-  // The input-gradient GEMM of a layer is told when a weight-gradient GEMM with a short K (small
-  // per-replica batch) runs next to it on the second stream; it then takes the kernel with the
-  // larger LDS footprint so that it keeps its share of every CU.  The hint follows the configured
-  // schedule, not the momentary one, so that the per-kernel timing pass measures the kernels the
-  // real step uses.
-  struct CorunScope {
-    mi_mlp* h;
-    explicit CorunScope(mi_mlp* h_) : h(h_) {}
-    ~CorunScope() { h->corun = false; }
-  } corun_scope(h);
-  const bool corun_cfg = !(h->flags & MI_FLAG_SERIAL_BACKWARD) && !crowded;
   for (int l = h->L - 1; l >= 0; --l) {
     if (paired) {
       if ((rc = op_backward_pair(h, l, s))) return rc;
       continue;
     }
-    h->corun = corun_cfg && h->B < 512;
     if ((rc = op_wgrad(h, l, s2, true))) return rc;
     if (dual) {
       MI_HIP(hipEventRecord(h->ev_wgrad[l], s2));

@@ -655,11 +655,9 @@ __device__ __forceinline__ void load_frag_swz(float (&frag)[TB][4], const float*
 // and epilogue are paid once per workgroup instead of once per replica, and the stores of a replica
 // drain under the next replica's MFMAs: the wait in front of the next ring barrier lets them stay
 // in flight (vmcnt retires in order, and the tile that barrier needs was requested before them).
-// Measured on 20 layers of 2048 x 2048 with 8 replicas of 256 rows: 129 us per launch against
-// 139 us for one workgroup per (replica, tile) -- but the whole step gets slower (8.1-8.5 ms against
-// 7.9 ms): the short workgroups of the plain kernel fill the prologue and epilogue gaps of the
-// input-gradient chain on the other stream, these long-lived ones only compete with it.  Hence
-// not part of the automatic choice; mi_set_gemm_variant(2, 35) selects it.
+// Measured on 20 layers of 2048 x 2048 with 8 replicas of 256 rows: 127-129 us per launch against
+// 139 us for one workgroup per (replica, tile).  How many replicas a workgroup should walk is a
+// matter of the whole step, see dispatch(): all 8 make the step slower, groups of 4 faster.
 template <int BM, int BN, int BK, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM, int STAGES,
           bool CHAIN = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
@@ -692,6 +690,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
   int tile_m, tile_n, bz;
   tile_of_block(p, tile_m, tile_n, bz);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
+  if (CHAIN) bz *= p.chain;  // the grid's batch index counts groups of p.chain consecutive entries
   float* __restrict__ C = p.C + (size_t)bz * p.batchC;
   float* __restrict__ colsum_out = COLSUM && p.colsum ? p.colsum + (size_t)bz * p.batchColsum + m0 : nullptr;
 
@@ -1088,9 +1087,9 @@ static hipError_t launch_dma(GemmArgs& p, int batch, hipStream_t s, bool exclusi
   constexpr size_t kExclusiveBytes = 84 * 1024;
   const size_t request = exclusive && lds_bytes < kExclusiveBytes ? kExclusiveBytes : lds_bytes;
   auto kern = gemm_f32_dma<BM, BN, BK, WM, WN, AK, BKM, EPI, COLSUM, STAGES, CHAIN>;
-  if (CHAIN) {  // the workgroup walks the batch itself: the grid covers one entry's tiles
-    p.chain = batch;
-    batch = 1;
+  if (CHAIN) {  // a workgroup walks p.chain consecutive batch entries itself: the grid covers batch / p.chain groups
+    if (p.chain <= 0 || batch % p.chain != 0) p.chain = batch;
+    batch /= p.chain;
   }
   static LdsOptIn opt_in;
   if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), request); e != hipSuccess) return e;
@@ -1132,27 +1131,39 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
   auto fits = [&](int bm, int bn, int bk) {
     return vec_ok && mask_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0;
   };
-  // variant 100 = automatic, and the caller runs a weight-gradient GEMM with a short K next to
-  // this one on a second stream (see below).
-  const bool corun = variant == 100;
-  if (corun) variant = 0;
+  const bool forced = variant != 0;
   if (variant == 0) {
     // Automatic choice.  From about one 128 x 128 tile per CU on, the direct-to-LDS kernels with a
     // ring of three buffers.  Measured on the benchmark configurations, whole step:
     //   * BK = 16 with the CU to itself (variant 34) everywhere, except
     //   * a weight gradient with a short K (small per-replica batch: few K steps, so prologue and
-    //     epilogue weigh most) takes BK = 16 at its natural 48 KB and shares CUs (variant 33), and
-    //   * the input-gradient GEMM that runs next to such a weight gradient takes BK = 32 (96 KB,
-    //     variant 31): one weight-gradient workgroup fits beside it, not two, which would slow the
-    //     chain of dependent input-gradient GEMMs that bounds the step.
+    //     epilogue weigh most) takes BK = 16 at its natural 48 KB and shares CUs; its replicas are
+    //     chained in groups (variant 35 with p.chain set) such that about two workgroups per CU
+    //     remain: config 4 (8 replicas of 256 rows, 256 tiles each) 7.89 -> 7.78 ms with groups of
+    //     4, but 8.0 ms with groups of 2 and 8.6 ms with all 8 in one workgroup, which leaves one
+    //     long-lived workgroup per CU and nothing to fill the gaps of the input-gradient chain on
+    //     the other stream.  (An earlier state gave the input-gradient GEMM next to such a weight
+    //     gradient BK = 32 and 96 KB; with the current kernels BK = 16 is better there too:
+    //     7.90 -> 7.76 ms.)
     // Smaller problems fall back to 128 x 64 and 64 x 64 tiles to get enough workgroups, the
     // smallest (config 1) to the split-K kernel.
     const long long tiles128 = (long long)(p.M / 128) * (p.N / 128) * batch;
     constexpr bool kWeightGradient = !AK && !BKM;
-    if (fits(128, 128, 32) && tiles128 >= 192 && corun) {
-      variant = 31;
-    } else if (fits(128, 128, 16) && tiles128 >= 192) {
-      variant = kWeightGradient && p.K < 512 ? 33 : 34;
+    if (fits(128, 128, 16) && tiles128 >= 192) {
+      variant = 34;
+      if (kWeightGradient && p.K < 512) {
+        variant = 33;
+        const long long tiles_entry = (long long)(p.M / 128) * (p.N / 128);
+        if (EPI == EPI_NONE && p.batchA == (long long)p.K * p.lda && p.batchB == (long long)p.K * p.ldb) {
+          int chain = 1;  // largest divisor of the replica count that leaves two workgroups per CU
+          for (int c = 2; c <= batch; ++c)
+            if (batch % c == 0 && tiles_entry * (batch / c) >= 512) chain = c;
+          if (chain > 1) {
+            variant = 35;
+            p.chain = chain;
+          }
+        }
+      }
     } else if (fits(128, 64, 32) && tiles128 * 2 >= 192) {
       variant = 11;
     } else if (fits(32, 32, 32) && (long long)(p.M / 64) * (p.N / 64) * batch < 192) {
@@ -1186,7 +1197,8 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
     case 31: if (fits(128, 128, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 32, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 33: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s); } break;
     case 34: if (fits(128, 128, 16)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3>(p, batch, s, true); } break;
-    case 35:
+    case 35: case 36: case 37:  // forced: 35 = all replicas in one workgroup, 36 / 37 = groups of 2 / 4; automatic: p.chain is set
+      if (forced) p.chain = variant == 35 ? 0 : variant == 36 ? 2 : 4;
       if constexpr (!AK && !BKM && EPI == EPI_NONE) {
         if (fits(128, 128, 16) && batch >= 1 && p.batchA == (long long)p.K * p.lda && p.batchB == (long long)p.K * p.ldb) {
           if (fused_colsum) *fused_colsum = COLSUM;
@@ -1203,7 +1215,7 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
 hipError_t sgemm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
                     int ldc, const float* bias, int relu, hipStream_t s, int variant) {
   // automatic choice: a layer of at most SKINNY_MAX outputs is matrix-vector work
-  if ((variant == 0 || variant == 100) && N <= SKINNY_MAX && K > 0)
+  if (variant == 0 && N <= SKINNY_MAX && K > 0)
     return sgemv_nt(M, N, K, A, lda, B, ldb, C, ldc, bias, relu, s);
   GemmArgs p{};
   p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
@@ -1213,7 +1225,7 @@ hipError_t sgemm_nt(int M, int N, int K, const float* A, int lda, const float* B
 
 hipError_t sgemm_nn(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
                     int ldc, const float* mask, int ldmask, hipStream_t s, int variant) {
-  if ((variant == 0 || variant == 100) && K <= SKINNY_MAX && K > 0)
+  if (variant == 0 && K <= SKINNY_MAX && K > 0)
     return sgemv_nn(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, s);
   GemmArgs p{};
   p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;

@@ -66,8 +66,7 @@ struct LdsOptIn {
   }
 };
 
-// `variant` selects a tile configuration of the MFMA kernel (0 = choose from the shape, 100 =
-// choose from the shape knowing that another GEMM runs concurrently on a second stream); it is
+// `variant` selects a tile configuration of the MFMA kernel (0 = choose from the shape); it is
 // exposed through mi_set_gemm_variant for tuning runs.
 hipError_t sgemm_nt(int M, int N, int K, const float* A, int lda, const float* B, int ldb, float* C,
                     int ldc, const float* bias, int relu, hipStream_t s, int variant);

@@ -96,7 +96,7 @@ GEMM_SHAPES = [
     # 16): the matrix-vector kernels, at the shapes of the reference's default last layer 1024 -> 1
     (4096, 1, 1024), (1, 1024, 1024), (4096, 1024, 1), (333, 16, 130), (16, 333, 130), (130, 333, 16), (50, 7, 1030),
 ]
-VARIANTS = [0, 8, 9, 10, 11, 12, 15, 16, 17, 21, 22, 30, 31, 33, 34, 35, 50]   # 35: weight gradient, one workgroup walks all replicas
+VARIANTS = [0, 8, 9, 10, 11, 12, 15, 16, 17, 21, 22, 30, 31, 33, 34, 35, 36, 37, 50]   # 35: weight gradient, one workgroup walks all replicas
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
