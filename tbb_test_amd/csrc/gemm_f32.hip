@@ -976,6 +976,91 @@ __global__ __launch_bounds__(256) void gemm_f32_splitk(GemmArgs p) {
   splitk_block<A_KMAJOR, B_KMAJOR, EPI, COLSUM>(p, blockIdx.x, blockIdx.z);
 }
 
+// The split-K kernel for two K-contiguous operands (the forward GEMM) with direct-to-LDS loads.
+// Loaded straight into registers, a K-contiguous fragment is 32-byte pieces of 32 different rows
+// per instruction; brought in through the LDS, a load instruction of a wavefront covers 4 rows x
+// 256 contiguous bytes.  Each wavefront owns its quarter of K and a private LDS region for it, so
+// there is no barrier in the loop: sub-blocks of 64 k (8 KB per operand) travel through two
+// buffers, the wavefront waits for its own loads (vmcnt) and multiplies from the LDS (rows of 256
+// bytes, 16-byte chunks XOR-swizzled with the row so that fragment reads touch every bank once).
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_f32_splitk_dma(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  constexpr int SW = 64;              // k per sub-block
+  constexpr int SB = 32 * SW;         // floats of one operand's sub-block
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, hi = lane >> 5;
+  const int tile_m = blockIdx.x / p.tiles_n, tile_n = blockIdx.x - tile_m * p.tiles_n;
+  const int m0 = tile_m * 32, n0 = tile_n * 32;
+  const int kq = p.K / 4, nsb = kq / SW;
+  float* region = smem + wave * (4 * SB);  // [buffer][A | B]
+  const unsigned lds_base = (unsigned)(size_t)((__attribute__((address_space(3))) const void*)region);
+  // load instruction j covers rows 4j .. 4j+3; lane i fills chunk position i % 16 of row 4j + i / 16
+  unsigned offa[8], offb[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int row = 4 * j + (lane >> 4), pos = lane & 15;
+    offa[j] = 4u * ((unsigned)row * (unsigned)p.lda + (unsigned)((pos ^ (row & 15)) * 4));
+    offb[j] = 4u * ((unsigned)row * (unsigned)p.ldb + (unsigned)((pos ^ (row & 15)) * 4));
+  }
+  const float* a_base = p.A + (size_t)m0 * p.lda + (size_t)wave * kq;
+  const float* b_base = p.B + (size_t)n0 * p.ldb + (size_t)wave * kq;
+  auto issue = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) load_to_lds_f32(a_base, offa[j], lds_base + 4u * (unsigned)(buf * 2 * SB + j * 256));
+#pragma unroll
+    for (int j = 0; j < 8; ++j) load_to_lds_f32(b_base, offb[j], lds_base + 4u * (unsigned)(buf * 2 * SB + SB + j * 256));
+    a_base += SW;
+    b_base += SW;
+  };
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+  issue(0);
+  if (nsb > 1) issue(1);
+  for (int sb = 0; sb < nsb; ++sb) {
+    const int cur = sb & 1;
+    if (sb + 1 < nsb) __builtin_amdgcn_s_waitcnt(vmcnt_only(16));  // the younger sub-block may stay in flight
+    else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+    asm volatile("" ::: "memory");
+    const float* a_tile = region + cur * 2 * SB + l32 * SW;
+    const float* b_tile = a_tile + SB;
+#pragma unroll
+    for (int kk = 0; kk < SW / 8; ++kk) {
+      const int chunk = ((2 * kk + hi) ^ (l32 & 15)) * 4;
+      const f32x4 fa = *reinterpret_cast<const f32x4*>(a_tile + chunk);
+      const f32x4 fb = *reinterpret_cast<const f32x4*>(b_tile + chunk);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[q], fb[q], acc, 0, 0, 0);
+    }
+    if (sb + 2 < nsb) {
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this buffer's fragments are in registers
+      asm volatile("" ::: "memory");
+      issue(cur);
+    }
+  }
+  // add the four partial blocks in wavefront order, as the register-loading kernel does
+  __syncthreads();
+  float(*part)[16][64] = reinterpret_cast<float(*)[16][64]>(smem);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) part[wave][r][lane] = acc[r];
+  __syncthreads();
+  const int col = n0 + l32;
+  const float bias_v = (EPI == EPI_BIAS_RELU && p.bias) ? p.bias[col] : 0.0f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int r = 4 * wave + e;
+    float v = ((part[0][r][lane] + part[1][r][lane]) + part[2][r][lane]) + part[3][r][lane];
+    const int row = m0 + 8 * wave + 4 * hi + e;
+    if (EPI == EPI_BIAS_RELU) {
+      v += bias_v;
+      if (p.relu) v = v > 0.0f ? v : 0.0f;
+    }
+    p.C[(size_t)row * p.ldc + col] = v;
+  }
+}
+
 // The two backward GEMMs of one layer in one launch: the weight gradient (all replicas, bias
 // gradient fused) and the input gradient read the same dZ and depend on nothing of each other.  For
 // problems this small a step is a chain of launches of a few microseconds each, and one launch less
@@ -1108,6 +1193,18 @@ static hipError_t launch_splitk(GemmArgs& p, int batch, hipStream_t s) {
   return hipGetLastError();
 }
 
+template <int EPI>
+static hipError_t launch_splitk_dma(GemmArgs& p, hipStream_t s) {
+  constexpr size_t lds_bytes = 4 * 4 * 32 * 64 * sizeof(float);  // 4 wavefronts x 2 buffers x 2 operands x 8 KB
+  auto kern = gemm_f32_splitk_dma<EPI>;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) return e;
+  p.tiles_m = p.M / 32;
+  p.tiles_n = p.N / 32;
+  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n), dim3(256), lds_bytes, s, p);
+  return hipGetLastError();
+}
+
 template <bool AK, bool BKM, int EPI>
 static hipError_t launch_generic(GemmArgs& p, int batch, hipStream_t s) {
   dim3 grid((p.N + 63) / 64, (p.M + 63) / 64, batch);
@@ -1168,6 +1265,7 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
       variant = 11;
     } else if (fits(32, 32, 32) && (long long)(p.M / 64) * (p.N / 64) * batch < 192) {
       variant = 50;  // fewer 64 x 64 tiles than CUs: 32 x 32 tiles with K split over the wavefronts
+      if (AK && BKM && EPI != EPI_MASK && batch == 1 && p.K % 256 == 0) variant = 51;  // both operands K-contiguous: through the LDS
     } else if (fits(64, 64, 16)) {
       variant = 16;
     } else if (p.K > 0) {
@@ -1204,6 +1302,11 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
           if (fused_colsum) *fused_colsum = COLSUM;
           return launch_dma<128, 128, 16, 2, 4, AK, BKM, EPI, COLSUM, 3, true>(p, batch, s);
         }
+      }
+      break;
+    case 51:
+      if constexpr (AK && BKM && EPI != EPI_MASK && !COLSUM) {
+        if (fits(32, 32, 256) && batch == 1) return launch_splitk_dma<EPI>(p, s);
       }
       break;
     case 50: if (fits(32, 32, 32)) { if (fused_colsum) *fused_colsum = COLSUM; return launch_splitk<AK, BKM, EPI, COLSUM>(p, batch, s); } break;

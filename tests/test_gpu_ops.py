@@ -82,6 +82,8 @@ def run_tn(dZ, A, R, variant=0, with_colsum=True):
 GEMM_SHAPES = [
     (128, 128, 32), (256, 128, 64), (128, 256, 96), (512, 512, 512), (384, 640, 160),
     (64, 64, 32), (192, 64, 64),
+    # split-K kernel with direct-to-LDS loads (forward GEMM, K a multiple of 256): one, two and five sub-blocks per wavefront
+    (64, 96, 256), (512, 512, 512), (96, 64, 1280),
     # tile grids whose XCD-aware orders divide by something that is not a power of two:
     # 8 x 3 tiles (contiguous range per XCD), 32 x 24 tiles (super-tiles, 3 per row)
     (1024, 384, 64), (4096, 3072, 32),
@@ -96,7 +98,7 @@ GEMM_SHAPES = [
     # 16): the matrix-vector kernels, at the shapes of the reference's default last layer 1024 -> 1
     (4096, 1, 1024), (1, 1024, 1024), (4096, 1024, 1), (333, 16, 130), (16, 333, 130), (130, 333, 16), (50, 7, 1030),
 ]
-VARIANTS = [0, 8, 9, 10, 11, 12, 15, 16, 17, 21, 22, 30, 31, 33, 34, 35, 36, 37, 50]   # 35: weight gradient, one workgroup walks all replicas
+VARIANTS = [0, 8, 9, 10, 11, 12, 15, 16, 17, 21, 22, 30, 31, 33, 34, 35, 36, 37, 50, 51]   # 35: weight gradient, one workgroup walks all replicas
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
