@@ -89,6 +89,10 @@ struct mi_mlp {
   // weight gradient of the last layer reads it every step; the rotation buffers get overwritten)
   uint16_t* dyT = nullptr;
   bool dyT_valid = false;
+  // bf16 only: column sums of dZ_l per block of 128 rows, written by the epilogue of the GEMM that
+  // produced dZ_l (slot l % ndz, [MB / 128][max N] floats); folded into the bias gradient by op_wgrad
+  std::vector<float*> colpart;
+  std::vector<char> colpart_valid;
   std::vector<void*> acts;    // L+1 buffers [MB x nf[l]], fp32 or bf16
   void* dy = nullptr;         // upstream gradient [MB x nf[L]]
   std::vector<void*> dz;      // [ndz] buffers of [MB x max width]
@@ -272,8 +276,13 @@ int op_wgrad(mi_mlp* h, int l, hipStream_t s, bool with_bias) {
     if (e == hipSuccess)
       e = mi::hgemm_nt(h->R, nout, nin, B, dzt, B, (long long)nout * B, h->actsT[l], B, (long long)nin * B,
                        const_cast<float*>(g0), nin, (long long)h->stride, 0, nullptr, 0, nullptr, 0, s, g_hvariant);
-    if (e == hipSuccess && with_bias)
-      e = mi::rowsum_bf16(h->R, nout, B, dzt, B, (long long)nout * B, h->grads + h->boff[l], (long long)h->stride, s);
+    if (e == hipSuccess && with_bias) {
+      // bias gradient: from the column sums the producing GEMM left behind, else a pass over dZ^T
+      if (l < h->L - 1 && h->colpart_valid[l % h->ndz] && B % 128 == 0)
+        e = mi::colsum_fold(h->R, nout, B / 128, h->colpart[l % h->ndz], h->grads + h->boff[l], (long long)h->stride, s);
+      else
+        e = mi::rowsum_bf16(h->R, nout, B, dzt, B, (long long)nout * B, h->grads + h->boff[l], (long long)h->stride, s);
+    }
   }
   if (e != hipSuccess) return hip_fail(e, "weight-gradient GEMM launch");
   return ts.finish();
@@ -307,12 +316,16 @@ int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
                      h->params + h->woff[l], h->nf[l], (float*)out, h->nf[l], (const float*)mask, h->nf[l], s,
                      g_variant[1]);
   } else {
-    bool wrote = false;
+    bool wrote = false, wrote_cs = false;
     uint16_t* ct = (l > 0) ? h->dzT[(l - 1) % h->ndz] : nullptr;  // dZ_{l-1}^T for the weight gradient of layer l-1
+    float* cp = (l > 0 && h->B % 128 == 0) ? h->colpart[(l - 1) % h->ndz] : nullptr;  // and its column sums
     e = mi::hgemm_nt(1, h->MB, h->nf[l], h->nf[l + 1], (const uint16_t*)dz_of_layer(h, l), h->nf[l + 1], 0,
                      h->params16T + h->woff[l], h->nf[l + 1], 0, out, h->nf[l], 0, mask ? 2 : 3, nullptr, 0,
-                     (const uint16_t*)mask, h->nf[l], s, g_hvariant, ct, h->B, &wrote);
-    if (l > 0) h->dzT_fused[(l - 1) % h->ndz] = wrote;
+                     (const uint16_t*)mask, h->nf[l], s, g_hvariant, ct, h->B, &wrote, cp, &wrote_cs);
+    if (l > 0) {
+      h->dzT_fused[(l - 1) % h->ndz] = wrote;
+      h->colpart_valid[(l - 1) % h->ndz] = wrote_cs;
+    }
   }
   if (e != hipSuccess) return hip_fail(e, "input-gradient GEMM launch");
   return ts.finish();
@@ -390,8 +403,8 @@ __global__ __launch_bounds__(256) void mask_copy_kernel(float* __restrict__ dst,
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step)
     dst[i] = act[i] > 0.0f ? g[i] : 0.0f;
 }
-// the same on bf16 words: positive = sign bit clear and not zero (a NaN output keeps the gradient,
-// as the fp32 comparison drops it; outputs of the forward GEMM are finite)
+// the same on bf16 words, compared after widening to fp32 (so zeros, negatives and NaN drop the
+// gradient exactly as in the fp32 kernel)
 __global__ __launch_bounds__(256) void mask_copy_bf16_kernel(uint16_t* __restrict__ dst, const uint16_t* __restrict__ g,
                                                              const uint16_t* __restrict__ act, size_t n) {
   const size_t step = (size_t)gridDim.x * blockDim.x;
@@ -938,6 +951,9 @@ int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_repli
     h->dzT_fused.assign(h->ndz, 0);
     for (int i = 0; i < h->ndz; ++i) alloc((void**)&h->dzT[i], (size_t)h->MB * h->maxw() * 2);
     alloc((void**)&h->dyT, (size_t)h->MB * h->nf[L] * 2);
+    h->colpart.assign(h->ndz, nullptr);
+    h->colpart_valid.assign(h->ndz, 0);
+    for (int i = 0; i < h->ndz; ++i) alloc((void**)&h->colpart[i], ((size_t)h->MB / 128 + 1) * h->maxw() * 4);
     h->actsT_fused.assign(L, 0);
     size_t wmax = 0;
     for (int l = 0; l < L; ++l) wmax = std::max(wmax, (size_t)h->nf[l] * h->nf[l + 1]);
@@ -1002,6 +1018,7 @@ int mi_mlp_destroy(mi_mlp* h) {
   for (auto a : h->actsT) (void)hipFree(a);
   for (auto a : h->dzT) (void)hipFree(a);
   (void)hipFree(h->dyT);
+  for (auto a : h->colpart) (void)hipFree(a);
   for (void* a : h->acts) (void)hipFree(a);
   (void)hipFree(h->dy);
   for (void* a : h->dz) (void)hipFree(a);

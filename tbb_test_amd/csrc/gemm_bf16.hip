@@ -56,6 +56,11 @@ struct HGemmArgs {
   int ct_rows;
   // guarded instances: whether A / B may be read with 16-byte vector loads
   int vec_a, vec_b;
+  // optional third output (bf16 epilogues of the 256 x 256 kernels): column sums of the values
+  // written, per wavefront tile of 128 rows -- colsum_part[row / 128][col], N floats per row block.
+  // Folded over a replica's row blocks they are the bias gradient of the layer whose dZ this GEMM
+  // produces, which saves a separate pass over that dZ.
+  float* colsum_part;
 };
 
 __device__ __forceinline__ u16 f2bf(float f) {
@@ -127,6 +132,7 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
   float* __restrict__ cf = reinterpret_cast<float*>(p.C) + (size_t)blockIdx.z * p.batchC;
   u16* __restrict__ ch = reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC;
   unsigned pk[TM][TN][8];  // bf16 results, two rows per register: (4g, 4g+1) and (4g+2, 4g+3)
+
   const unsigned mask_lds_addr = MASK_LDS ? (unsigned)(size_t)((__attribute__((address_space(3))) const void*)mask_lds) : 0u;
   (void)mask_lds_addr;
   if constexpr (EPI == EPH_F32) {
@@ -185,6 +191,23 @@ __device__ __forceinline__ void store_tile_h(const HGemmArgs& p, f32x16 (&acc)[T
           if (second_row) ch[(size_t)(row + 1) * p.ldc + col] = (u16)(two >> 16);
         }
       }
+    }
+  }
+  if (EPI != EPH_F32 && !GUARD && p.colsum_part) {
+    // the two lane halves hold different rows of the same column; one row block = this wavefront's TM * 32 rows
+    // (summed from the packed results after the stores, so that nothing extra is live in the loop
+    // above: the values added are the rounded ones, i.e. exactly what was written)
+    float* part = p.colsum_part + (size_t)(row0 / (TM * 32)) * p.N;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      float c = 0.0f;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int rp = 0; rp < 8; ++rp)
+          c += __uint_as_float(pk[i][j][rp] << 16) + __uint_as_float(pk[i][j][rp] & 0xffff0000u);
+      const float total = c + __shfl_xor(c, 32, 64);
+      if (hi == 0) part[col0 + j * 32] = total;
     }
   }
   if (EPI == EPH_F32 || GUARD || !p.Ct) return;
@@ -768,7 +791,7 @@ static hipError_t launch_dma(HGemmArgs& p, int batch, hipStream_t s) {
 }
 
 template <int EPI>
-static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant, bool* wrote_ct) {
+static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant, bool* wrote_ct, bool* wrote_colsum) {
   if (wrote_ct) *wrote_ct = p.Ct != nullptr && EPI != EPH_F32;
   if (p.M <= 0 || p.N <= 0 || batch <= 0) return hipSuccess;
   auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
@@ -794,6 +817,9 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
   }
   p.vec_a = al16(p.A) && p.lda % 8 == 0 && p.batchA % 8 == 0;
   p.vec_b = al16(p.B) && p.ldb % 8 == 0 && p.batchB % 8 == 0;
+  // column-sum partials come from the 256 x 256 direct-load kernels (wavefront tiles of 128 rows) only
+  if (p.colsum_part && !((variant == 13 || variant == 19) && EPI != EPH_F32 && batch == 1 && p.M % 128 == 0)) p.colsum_part = nullptr;
+  if (wrote_colsum) *wrote_colsum = p.colsum_part != nullptr;
   {  // the tile height decides whether the transposed output is possible; if not, drop it
     const int bm = (variant == 3 || variant == 17) ? 128 : variant == 5 ? 64 : 256;
     if (want_ct && (EPI == EPH_F32 || variant == 21 || variant == 22 || !ct_ok(bm))) {
@@ -813,7 +839,9 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     default: break;
   }
   if (wrote_ct) *wrote_ct = false;  // the any-shape kernel has no transposed output
+  if (wrote_colsum) *wrote_colsum = false;
   p.Ct = nullptr;
+  p.colsum_part = nullptr;
   launch_kernel((gemm_bf16_generic<EPI>), dim3((p.N + 15) / 16, (p.M + 15) / 16, batch), dim3(256), 0, s, p);
   return hipGetLastError();
 }
@@ -823,18 +851,39 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
 hipError_t hgemm_nt(int batch, int M, int N, int K, const uint16_t* A, int lda, long long batchA, const uint16_t* B,
                     int ldb, long long batchB, void* C, int ldc, long long batchC, int out_kind, const float* bias,
                     int relu, const uint16_t* mask, int ldmask, hipStream_t s, int variant, uint16_t* Ct, int ct_rows,
-                    bool* wrote_ct) {
+                    bool* wrote_ct, float* colsum_part, bool* wrote_colsum) {
   HGemmArgs p{};
   p.Ct = Ct; p.ct_rows = ct_rows;
+  p.colsum_part = colsum_part;
   p.M = M; p.N = N; p.K = K; p.A = A; p.B = B; p.C = C; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.batchA = batchA; p.batchB = batchB; p.batchC = batchC;
   p.bias = bias; p.relu = relu; p.mask = mask; p.ldmask = ldmask;
   switch (out_kind) {
-    case 0: return dispatch_h<EPH_F32>(p, batch, s, variant, wrote_ct);
-    case 1: return dispatch_h<EPH_BIAS_RELU>(p, batch, s, variant, wrote_ct);
-    case 2: return dispatch_h<EPH_MASK>(p, batch, s, variant, wrote_ct);
-    default: return dispatch_h<EPH_BF16>(p, batch, s, variant, wrote_ct);
+    case 0: return dispatch_h<EPH_F32>(p, batch, s, variant, wrote_ct, wrote_colsum);
+    case 1: return dispatch_h<EPH_BIAS_RELU>(p, batch, s, variant, wrote_ct, wrote_colsum);
+    case 2: return dispatch_h<EPH_MASK>(p, batch, s, variant, wrote_ct, wrote_colsum);
+    default: return dispatch_h<EPH_BF16>(p, batch, s, variant, wrote_ct, wrote_colsum);
   }
+}
+
+// ---- bias gradient from the column-sum partials of the GEMM that produced dZ ------------------------
+// out[r * stride_out + c] = sum over the `blocks` row blocks of replica r of part[(r * blocks + q) * N + c],
+// in block order (deterministic).
+__global__ __launch_bounds__(256) void colsum_fold_kernel(float* __restrict__ out, long long stride_out,
+                                                          const float* __restrict__ part, int N, int blocks) {
+  const int c = blockIdx.x * 256 + threadIdx.x, r = blockIdx.y;
+  if (c >= N) return;
+  const float* q = part + (size_t)r * blocks * N + c;
+  float v = 0.0f;
+  for (int b = 0; b < blocks; ++b) v += q[(size_t)b * N];
+  out[(size_t)r * stride_out + c] = v;
+}
+
+hipError_t colsum_fold(int R, int N, int blocks_per_replica, const float* part, float* out, long long stride_out,
+                       hipStream_t s) {
+  if (R <= 0 || N <= 0) return hipSuccess;
+  launch_kernel(colsum_fold_kernel, dim3((N + 255) / 256, R), dim3(256), 0, s, out, stride_out, part, N, blocks_per_replica);
+  return hipGetLastError();
 }
 
 // ---- batched transpose: dst[z][c][r] = src[z][r][c], 16-bit elements, 64 x 64 tiles through LDS ----

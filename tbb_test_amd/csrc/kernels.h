@@ -124,10 +124,16 @@ hipError_t reduce_sgd_tiled(float* W, uint16_t* W16, uint16_t* W16T, const float
 // ReLU, 2 bf16 zeroed where mask (bf16) <= 0, 3 bf16 plain.  Ct (bf16 output kinds, batch 1): the
 // result is also written transposed per group of ct_rows rows, Ct[row / ct_rows][col][row % ct_rows];
 // *wrote_ct tells whether the kernel that was chosen could do that (else the caller transposes).
+// colsum_part (bf16 output kinds, batch 1): the kernel also writes column sums of its output per block
+// of 128 rows, colsum_part[row / 128][col] (N floats per block); *wrote_colsum tells whether the
+// chosen kernel did.  colsum_fold adds a replica's blocks up: the bias gradient of the layer whose
+// dZ the GEMM produced.
 hipError_t hgemm_nt(int batch, int M, int N, int K, const uint16_t* A, int lda, long long batchA, const uint16_t* B,
                     int ldb, long long batchB, void* C, int ldc, long long batchC, int out_kind, const float* bias,
                     int relu, const uint16_t* mask, int ldmask, hipStream_t s, int variant, uint16_t* Ct = nullptr,
-                    int ct_rows = 0, bool* wrote_ct = nullptr);
+                    int ct_rows = 0, bool* wrote_ct = nullptr, float* colsum_part = nullptr, bool* wrote_colsum = nullptr);
+hipError_t colsum_fold(int R, int N, int blocks_per_replica, const float* part, float* out, long long stride_out,
+                       hipStream_t s);
 // dst[z][c][r] = src[z][r][c] for 16-bit elements
 // mfma_probe.hip: TFLOP/s of a register-resident MFMA loop (operands: 0 zeros, 1 ones, 2 random)
 hipError_t probe_mfma_rate(bool bf16, int operands, double* tflops, hipStream_t s);
