@@ -222,7 +222,9 @@ int mi_mlp_create(mi_mlp** h, int L, const int* nfeatures, int batch_per_replica
 int mi_mlp_destroy(mi_mlp* h);
 
 /* Host -> device uploads.  ld in elements; b may be NULL (bias = 0).  Stand in for
- * init_matrices(), mlp_bench_common.cc:16-33. */
+ * init_matrices(), mlp_bench_common.cc:16-33.  bf16 models convert on the device and also make the
+ * K-contiguous copies their GEMMs read (W^T at mi_mlp_set_weights, the per-replica X^T and dY^T at
+ * mi_mlp_set_input / mi_mlp_set_dy), so that a step moves none of these again. */
 int mi_mlp_set_weights(mi_mlp* h, int l, const float* W, int ld, const float* b);
 int mi_mlp_set_input(mi_mlp* h, const float* X, int ld);
 int mi_mlp_set_dy(mi_mlp* h, const float* dY, int ld);
