@@ -96,6 +96,7 @@ def main():
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--flat-update", action="store_true",
                     help="one update launch at the end of the step instead of per-layer updates on the second stream")
+    ap.add_argument("--hvariant", type=int, default=0, help="tuning: forced bf16 GEMM tile variant")
     ap.add_argument("--variants", default="", help="tuning: forced GEMM tile variants 'nt,nn,tn'")
     ap.add_argument("--serial-backward", action="store_true", help="whole backward pass on one stream")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg (0 = skip)")
@@ -117,6 +118,8 @@ def main():
     X, Ws, dY = hostlib.init_problem(nf, B, R, args.seed)
     flags = (0 if args.flat_update else capi.FLAG_PER_LAYER_UPDATE) | (capi.FLAG_SERIAL_BACKWARD if args.serial_backward else 0)
     h = capi.MlpHandle(nf, B, R, dtype=capi.MI_BF16 if dtype == "bf16" else capi.MI_F32, flags=flags)
+    if args.hvariant:
+        capi.check(capi.lib().mi_set_hgemm_variant(args.hvariant))
     if args.variants:
         for kind, v in enumerate(int(x) for x in args.variants.split(",")):
             capi.check(capi.lib().mi_set_gemm_variant(kind, v))

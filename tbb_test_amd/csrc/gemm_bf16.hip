@@ -498,7 +498,7 @@ __device__ __forceinline__ void ring_barrier() {
 
 // The lambdas are always_inline: left to its cost model the compiler keeps the K-step lambdas of
 // large instantiations as real functions, and the accumulators they capture then live in memory.
-template <int BM, int BN, int BK, int WM, int WN, int EPI, int STAGES>
+template <int BM, int BN, int BK, int WM, int WN, int EPI, int STAGES, int PRIO = 0>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
   constexpr int NW = WM * WN;
   constexpr int WTM = BM / WM, WTN = BN / WN;
@@ -602,12 +602,19 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma(HGemmArgs p) {
 
   const int nk = p.K / BK;
   bf16x8 fa[2][TM], fb[2][TN];
+  // PRIO = 1: a wavefront raises its issue priority for the MFMAs of a chunk and drops it for the
+  // fragment reads and tile loads in between.  The two wavefronts of a SIMD then fall into
+  // alternation (one multiplies while the other fetches) instead of competing for the MFMA pipe
+  // with half-issued chunks: 3-3.5 % on the two-buffer BK = 64 kernel, nothing on the BK = 32 ring
+  // and a small loss on the fp32 kernel, which therefore keep equal priorities.
   auto multiply = [&](int fc) __attribute__((always_inline)) {
+    if (PRIO == 1) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[fc][i], fb[fc][j], acc[i][j], 0, 0, 0);
+    if (PRIO == 1) __builtin_amdgcn_s_setprio(0);
   };
   if constexpr (STAGES == 2) {
     // Two buffers (what fits when BK = 64 makes a 256 x 256 tile 64 KB).  BK = 64 rows are whole
@@ -777,11 +784,11 @@ static hipError_t launch_h(HGemmArgs& p, int batch, hipStream_t s) {
   return hipGetLastError();
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int EPI, int STAGES>
+template <int BM, int BN, int BK, int WM, int WN, int EPI, int STAGES, int PRIO = 0>
 static hipError_t launch_dma(HGemmArgs& p, int batch, hipStream_t s) {
   constexpr size_t lds_bytes = STAGES * (size_t)(BM + BN) * BK * sizeof(u16);
   static_assert(lds_bytes <= 160 * 1024, "tile does not fit the 160 KB of LDS");
-  auto kern = gemm_bf16_dma<BM, BN, BK, WM, WN, EPI, STAGES>;
+  auto kern = gemm_bf16_dma<BM, BN, BK, WM, WN, EPI, STAGES, PRIO>;
   static LdsOptIn opt_in;
   if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) return e;
   p.tiles_m = p.M / BM;
@@ -818,10 +825,10 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
   p.vec_a = al16(p.A) && p.lda % 8 == 0 && p.batchA % 8 == 0;
   p.vec_b = al16(p.B) && p.ldb % 8 == 0 && p.batchB % 8 == 0;
   // column-sum partials come from the 256 x 256 direct-load kernels (wavefront tiles of 128 rows) only
-  if (p.colsum_part && !((variant == 13 || variant == 19) && EPI != EPH_F32 && batch == 1 && p.M % 128 == 0)) p.colsum_part = nullptr;
+  if (p.colsum_part && !((variant == 13 || variant == 19 || variant == 25) && EPI != EPH_F32 && batch == 1 && p.M % 128 == 0)) p.colsum_part = nullptr;
   if (wrote_colsum) *wrote_colsum = p.colsum_part != nullptr;
   {  // the tile height decides whether the transposed output is possible; if not, drop it
-    const int bm = (variant == 3 || variant == 17) ? 128 : variant == 5 ? 64 : 256;
+    const int bm = (variant == 3 || variant == 17) ? 128 : variant == 5 ? 64 : 256;  // (variants 13, 19, 25: 256)
     if (want_ct && (EPI == EPH_F32 || variant == 21 || variant == 22 || !ct_ok(bm))) {
       p.Ct = nullptr;
       if (wrote_ct) *wrote_ct = false;
@@ -833,7 +840,8 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     case 5: if (fits(64, 64, 32)) return launch_h<64, 64, 32, 2, 2, EPI>(p, batch, s); break;
     case 13: if (fits(256, 256, 32)) return launch_dma<256, 256, 32, 2, 4, EPI, 4>(p, batch, s); break;
     case 17: if (fits(128, 128, 32)) return launch_dma<128, 128, 32, 2, 2, EPI, 4>(p, batch, s); break;
-    case 19: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2>(p, batch, s); break;
+    case 19: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2, 1>(p, batch, s); break;
+    case 25: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2, 0>(p, batch, s); break;
     case 21: if (p.K > 0) return launch_h<128, 128, 32, 2, 2, EPI, 1, 3, true>(p, batch, s); break;
     case 22: if (p.K > 0) return launch_h<64, 64, 32, 2, 2, EPI, 1, 3, true>(p, batch, s); break;
     default: break;
