@@ -25,83 +25,10 @@
 #include <type_traits>
 #include <utility>
 
+#include "gemm_bf16_common.h"
 #include "kernels.h"
 
 namespace mi {
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef unsigned short u16;
-
-enum EpilogueH { EPH_F32 = 0, EPH_BIAS_RELU = 1, EPH_MASK = 2, EPH_BF16 = 3 };
-
-struct HGemmArgs {
-  int M, N, K;
-  const u16* A;
-  const u16* B;
-  void* C;  // bf16 or fp32, see the epilogue
-  int lda, ldb, ldc;
-  long long batchA, batchB, batchC;  // element offsets per blockIdx.z
-  const float* bias;
-  int relu;
-  const u16* mask;  // bf16 [M x N]: result zeroed where mask <= 0
-  int ldmask;
-  int tiles_m, tiles_n;
-  // optional second output (bf16 epilogues): the same values transposed per group of ct_rows
-  // rows, Ct[(row / ct_rows)][col][row % ct_rows] with row stride ct_rows and N * ct_rows elements
-  // per group -- the K-contiguous per-replica copy the weight-gradient GEMM reads
-  u16* Ct;
-  int ct_rows;
-  // guarded instances: whether A / B may be read with 16-byte vector loads
-  int vec_a, vec_b;
-  // optional third output (bf16 epilogues of the 256 x 256 kernels): column sums of the values
-  // written, per wavefront tile of 128 rows -- colsum_part[row / 128][col], N floats per row block.
-  // Folded over a replica's row blocks they are the bias gradient of the layer whose dZ this GEMM
-  // produces, which saves a separate pass over that dZ.
-  float* colsum_part;
-};
-
-__device__ __forceinline__ u16 f2bf(float f) {
-  unsigned int u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (u16)(u >> 16);
-}
-__device__ __forceinline__ float bf2f(u16 h) { return __uint_as_float((unsigned int)h << 16); }
-
-__device__ __forceinline__ void lds_barrier_h() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-// Maps the flat workgroup index to a C tile.  Workgroups are handed to the 8 XCDs round-robin
-// (id % 8), each XCD has a private 4 MB L2, and about 32 workgroups (one per CU) of an XCD run at
-// the same time.
-//   * Large grids (tile counts divisible as needed): the grid is cut into super-tiles of 4 x 8
-//     tiles; XCD x owns super-tiles x, x+8, ... and walks each row by row, so the 32 tiles it
-//     runs together share 4 A panels and 8 B panels -- 12 panel slices per K step from the
-//     fabric instead of the 33 a single tile row needs.
-//   * Otherwise, if the tile count is a multiple of 8: XCD x gets the contiguous range
-//     [x*T/8, (x+1)*T/8) of the row-major order (tiles of one row share their A panel).
-//   * Otherwise the identity.
-__device__ __forceinline__ void tile_of_workgroup(int id, int tiles_m, int tiles_n, int& tm, int& tn) {
-  const int total = tiles_m * tiles_n;
-  if ((tiles_m & 3) == 0 && (tiles_n & 7) == 0 && (total & 255) == 0) {
-    const int xcd = id & 7, j = id >> 3;
-    const int super = (j >> 5) * 8 + xcd, within = j & 31;
-    const int super_cols = tiles_n >> 3;
-    tm = (super / super_cols) * 4 + (within >> 3);
-    tn = (super % super_cols) * 8 + (within & 7);
-    return;
-  }
-  if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
-  tm = id / tiles_n;
-  tn = id - tm * tiles_n;
-}
-
 // Writes a wavefront's TM x TN accumulator blocks (32 x 32 each) with the epilogue EPI.  Lane l,
 // register r of a block hold row 8*(r/4) + 4*(l/32) + r%4, column l%32.
 //
@@ -463,39 +390,6 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_mfma(HGemmArgs p) {
 // Written this way the compiler does not track the load at all; the kernel waits on vmcnt itself
 // (its own waits can only become longer through the extra loads in flight, never shorter, because
 // vmcnt retires in order).  m0 carries the wave-uniform LDS byte address.
-__device__ __forceinline__ void load_to_lds(const u16* uniform_base, unsigned lane_byte_offset, unsigned lds_byte_addr) {
-  const unsigned lds_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr);
-  const unsigned long long b = reinterpret_cast<unsigned long long>(uniform_base);
-  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b), hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
-  const unsigned long long sbase = ((unsigned long long)hi << 32) | lo;
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :
-               : "s"(lds_addr), "v"(lane_byte_offset), "s"(sbase)
-               : "memory", "m0");
-}
-
-template <int... S, class F>
-__device__ __forceinline__ void static_for_h_impl(std::integer_sequence<int, S...>, F&& f) {
-  (f(std::integral_constant<int, S>{}), ...);
-}
-template <int N, class F>
-__device__ __forceinline__ void static_for_h(F&& f) {
-  static_for_h_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
-}
-
-// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
-// expcnt 6:4, lgkmcnt 11:8; the other counters at their maximum = no wait).
-constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x70 | 0xf00; }
-
-// Barrier of the ring: no LDS-counter wait is attached (nothing was written with ds_write, and a
-// buffer is refilled only after the MFMAs that consumed its last fragments, i.e. after those reads
-// returned); the empty asm statements keep the compiler from moving LDS reads across it.
-__device__ __forceinline__ void ring_barrier() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
-
 // The lambdas are always_inline: left to its cost model the compiler keeps the K-step lambdas of
 // large instantiations as real functions, and the accumulators they capture then live in memory.
 template <int BM, int BN, int BK, int WM, int WN, int EPI, int STAGES, int PRIO = 0>
@@ -814,7 +708,7 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     // 256 x 256 tiles with 8 wavefronts and direct-to-LDS loads once they cover the CUs (whole
     // 128-byte lines per row when K allows BK = 64), else smaller tiles for more workgroups
     const long long t256 = (long long)(p.M / 256) * (p.N / 256) * batch;
-    if (fits(256, 256, 64) && t256 >= 256) variant = 19;
+    if (fits(256, 256, 64) && t256 >= 256) variant = 27;  // falls back to 19 below if C or the mask is not 16-byte aligned
     else if (fits(256, 256, 32) && t256 >= 256) variant = 13;
     else if (fits(128, 128, 32) && (long long)(p.M / 128) * (p.N / 128) * batch >= 128) variant = 3;
     else if (fits(64, 64, 32)) variant = 5;
@@ -822,13 +716,20 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
       variant = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * batch >= 192 ? 21 : 22;
     else variant = -1;
   }
+  // the 16x16x32 kernel writes C and reads the mask in 16-byte pieces
+  auto x32_ok = [&]() {
+    const int per16 = EPI == EPH_F32 ? 4 : 8;
+    return fits(256, 256, 64) && al16(p.C) && p.ldc % per16 == 0 && p.batchC % per16 == 0 &&
+           (EPI != EPH_MASK || (al16(p.mask) && p.ldmask % 8 == 0));
+  };
+  if ((variant == 27 || variant == 28) && !x32_ok()) variant = 19;
   p.vec_a = al16(p.A) && p.lda % 8 == 0 && p.batchA % 8 == 0;
   p.vec_b = al16(p.B) && p.ldb % 8 == 0 && p.batchB % 8 == 0;
   // column-sum partials come from the 256 x 256 direct-load kernels (wavefront tiles of 128 rows) only
-  if (p.colsum_part && !((variant == 13 || variant == 19 || variant == 25) && EPI != EPH_F32 && batch == 1 && p.M % 128 == 0)) p.colsum_part = nullptr;
+  if (p.colsum_part && !((variant == 13 || variant == 19 || variant == 25 || variant == 27 || variant == 28) && EPI != EPH_F32 && batch == 1 && p.M % 128 == 0)) p.colsum_part = nullptr;
   if (wrote_colsum) *wrote_colsum = p.colsum_part != nullptr;
   {  // the tile height decides whether the transposed output is possible; if not, drop it
-    const int bm = (variant == 3 || variant == 17) ? 128 : variant == 5 ? 64 : 256;  // (variants 13, 19, 25: 256)
+    const int bm = (variant == 3 || variant == 17) ? 128 : variant == 5 ? 64 : 256;  // (variants 13, 19, 25, 27, 28: 256)
     if (want_ct && (EPI == EPH_F32 || variant == 21 || variant == 22 || !ct_ok(bm))) {
       p.Ct = nullptr;
       if (wrote_ct) *wrote_ct = false;
@@ -842,6 +743,8 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     case 17: if (fits(128, 128, 32)) return launch_dma<128, 128, 32, 2, 2, EPI, 4>(p, batch, s); break;
     case 19: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2, 1>(p, batch, s); break;
     case 25: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2, 0>(p, batch, s); break;
+    case 27: return launch_x32(p, batch, EPI, true, s);
+    case 28: return launch_x32(p, batch, EPI, false, s);
     case 21: if (p.K > 0) return launch_h<128, 128, 32, 2, 2, EPI, 1, 3, true>(p, batch, s); break;
     case 22: if (p.K > 0) return launch_h<64, 64, 32, 2, 2, EPI, 1, 3, true>(p, batch, s); break;
     default: break;

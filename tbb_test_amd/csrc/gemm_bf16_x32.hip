@@ -1,0 +1,346 @@
+// bf16 GEMM for gfx950 on v_mfma_f32_16x16x32_bf16: C[M,N] = A[M,K] * B[N,K]^T, both operands
+// K-contiguous, fp32 accumulation -- the kernel of the large GEMMs of the MLP step (reference call
+// sites mlp_omp.cc:474-488, 565-580, 657-671).
+//
+// Why this instruction.  The bf16 matrix cores of this device are power-limited: a register-resident
+// loop of 32x32x16 MFMAs sustains about 1 800 TFLOP/s on random operands, the same loop of 16x16x32
+// MFMAs about 2 050 (a 16 x 16 block accumulates 32 k per instruction: half the accumulator traffic
+// per flop).  The clock the GEMM runs at follows.
+//
+// Tile 256 x 256 x 64, eight wavefronts of 128 (m) x 64 (n), two LDS buffers filled by direct
+// global -> LDS loads, one barrier per K step: the ring of gemm_bf16_dma (gemm_bf16.hip) with other
+// fragments.  A step is four sub-chunks of 16 MFMAs: K chunk kc = 0, 1 (32 k each) times the lower
+// and upper four 16-row blocks of the wavefront's m range; the n-side fragments of a K chunk stay
+// in registers for both halves.
+//
+// Orientation.  The MFMA's register-side index (row 4 * (lane / 16) + r of the 16 x 16 result) is
+// given to n and its lane-side index (lane % 16) to m, and the rows of the B tile are dealt to the
+// four n blocks so that a lane ends up with two runs of eight consecutive columns of one row of C
+// (columns 8q .. 8q+7 and 32 + 8q .. 32 + 8q+7 of the wavefront's 64, q = lane / 16):
+//   block ip, register-side index 4q + r  ->  column 32 * (ip / 2) + 8q + 4 * (ip % 2) + r.
+// The epilogue therefore writes C, and reads the ReLU mask, in 16-byte pieces per lane with no
+// shuffling (fp32 results: 32 contiguous bytes per lane).  The B tile's LDS swizzle is chosen for
+// that row order: the 16 lanes of a quarter-wave read rows 8q' + r' (+ multiples of 4 and 32),
+// swizzle = 2 * ((row / 8) % 4) + (row / 2) % 2 gives them 16 distinct 16-byte slots.
+//
+// The transposed per-replica copy (Ct) wants runs along m instead: it goes through the then idle
+// LDS, one private region per wavefront, as in gemm_bf16_dma.
+#include <hip/hip_runtime.h>
+
+#include "gemm_bf16_common.h"
+
+namespace mi {
+
+namespace {
+
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) const bf16x8 lds_frag;
+
+constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 4, NW = WM * WN;
+constexpr int WTM = BM / WM, WTN = BN / WN;   // 128 x 64 per wavefront
+constexpr int QB = WTM / 16, PB = WTN / 16;   // 8 lane-side (m) blocks, 4 register-side (n) blocks
+constexpr int A_ELEMS = BM * BK, B_ELEMS = BN * BK;
+constexpr int VPR = BK / 8;                   // 16-byte chunks per tile row (a whole 128-byte line)
+constexpr int RPI = 64 / VPR;                 // tile rows one load instruction of a wave fills
+constexpr int NIA = BM / (RPI * NW), NIB = BN / (RPI * NW);
+constexpr int INSTR = NIA + NIB;
+constexpr size_t LDS_BYTES = 2 * (size_t)(A_ELEMS + B_ELEMS) * sizeof(u16);  // 128 KB
+constexpr int STAGE_COL_BYTES = WTM * 2 + 8;  // one staged column of the transposed output + pad
+constexpr int STAGE_REGION = 32 * STAGE_COL_BYTES;
+static_assert((size_t)NW * STAGE_REGION <= LDS_BYTES, "staging must fit the ring");
+
+__device__ __forceinline__ int swz_a(int row) { return (row >> 1) & 7; }
+__device__ __forceinline__ int swz_b(int row) { return ((row >> 3) & 3) * 2 + ((row >> 1) & 1); }
+
+// Epilogue of one wavefront: acc[jq][ip] is the 16 x 16 block of rows row0 + 16 jq + lane % 16 and
+// the four columns described at the top of the file.
+template <int EPI>
+__device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][PB], int row0, int colw, int lane,
+                                          unsigned char* region) {
+  const int l16 = lane & 15, q = lane >> 4;
+  if constexpr (EPI == EPH_F32) {
+    float* __restrict__ cf = reinterpret_cast<float*>(p.C) + (size_t)blockIdx.z * p.batchC;
+#pragma unroll
+    for (int jq = 0; jq < QB; ++jq) {
+      float* dst = cf + (size_t)(row0 + 16 * jq + l16) * p.ldc + colw + 8 * q;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        *reinterpret_cast<f32x4*>(dst + 32 * h) = acc[jq][2 * h];
+        *reinterpret_cast<f32x4*>(dst + 32 * h + 4) = acc[jq][2 * h + 1];
+      }
+    }
+    return;
+  } else {
+    u16* __restrict__ ch = reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC;
+    u32x4 pk[QB][2];  // the rounded results: eight consecutive columns per register quadruple
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int col = colw + 32 * h + 8 * q;
+      float bias_v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) bias_v[e] = (EPI == EPH_BIAS_RELU && p.bias) ? p.bias[col + e] : 0.0f;
+#pragma unroll
+      for (int jq = 0; jq < QB; ++jq) {
+        const int row = row0 + 16 * jq + l16;
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = acc[jq][2 * h + (e >> 2)][e & 3];
+        if (EPI == EPH_BIAS_RELU) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            v[e] += bias_v[e];
+            if (p.relu) v[e] = v[e] > 0.0f ? v[e] : 0.0f;
+          }
+        } else if (EPI == EPH_MASK) {
+          const u32x4 mk = *reinterpret_cast<const u32x4*>(p.mask + (size_t)row * p.ldmask + col);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const u16 m = (u16)(mk[e >> 1] >> (16 * (e & 1)));
+            if (!(bf2f(m) > 0.0f)) v[e] = 0.0f;
+          }
+        }
+        u32x4 out;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const f32x2_t two = {v[2 * e], v[2 * e + 1]};
+          out[e] = __builtin_bit_cast(unsigned, __builtin_convertvector(two, bf16x2_t));  // round to nearest even
+        }
+        pk[jq][h] = out;
+        *reinterpret_cast<u32x4*>(ch + (size_t)row * p.ldc + col) = out;
+      }
+    }
+    if (p.colsum_part) {
+      // Column sums of the rounded values over the wavefront's 128 rows: a lane adds its eight rows
+      // in block order, the 16 lanes of a quarter-wave are folded with a fixed butterfly.
+      float* part = p.colsum_part + (size_t)(row0 / WTM) * p.N;
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float c = 0.0f;
+#pragma unroll
+          for (int jq = 0; jq < QB; ++jq) {
+            const unsigned two = pk[jq][h][e >> 1];
+            c += (e & 1) ? __uint_as_float(two & 0xffff0000u) : __uint_as_float(two << 16);
+          }
+#pragma unroll
+          for (int off = 1; off < 16; off <<= 1) c += __shfl_xor(c, off, 64);
+          if (l16 == 0) part[colw + 32 * h + 8 * q + e] = c;
+        }
+    }
+    if (!p.Ct) return;
+    // Transposed copy: the tile lies inside one row group (ct_rows is a multiple of the tile height).
+    // 32 columns at a time are staged [column][row] in the wavefront's LDS region (columns padded by
+    // 8 bytes) and read back as 16-byte chunks: a store instruction writes runs of 256 contiguous bytes.
+    const int group = row0 / p.ct_rows, m_local0 = row0 - group * p.ct_rows;
+    u16* __restrict__ ct = p.Ct + (size_t)group * p.N * p.ct_rows + m_local0;
+    // Neighbouring lanes hold neighbouring rows.  One exchange with lane ^ 1 turns a register (columns
+    // 2k, 2k+1 of one row) into (rows 2p, 2p+1 of one column): even lanes keep the even columns, odd
+    // lanes the odd ones, and the staging writes are 4 bytes instead of 2.
+    const bool odd = lane & 1;
+    const unsigned sel = odd ? 0x07060302u : 0x01000504u;  // bytes of {own (4-7), partner (0-3)}
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int jq = 0; jq < QB; ++jq)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const unsigned own = pk[jq][h][k];
+          const unsigned partner = (unsigned)__builtin_amdgcn_update_dpp(0, (int)own, 0xB1, 0xf, 0xf, false);  // lane ^ 1
+          // even lane: (own.lo, partner.lo) = rows (m, m+1) of column 2k; odd lane: (partner.hi, own.hi) = rows (m-1, m) of column 2k+1
+          const unsigned two = __builtin_amdgcn_perm(own, partner, sel);
+          *reinterpret_cast<unsigned*>(region + (8 * q + 2 * k + (lane & 1)) * STAGE_COL_BYTES + (16 * jq + (l16 & 14)) * 2) = two;
+        }
+      constexpr int CHUNKS = WTM / 8;  // 16-byte chunks per column
+#pragma unroll
+      for (int i = lane; i < 32 * CHUNKS; i += 64) {
+        const int c = i / CHUNKS, piece = i % CHUNKS;
+        // columns start at multiples of 8 bytes only: two 8-byte LDS reads per 16-byte global store
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(region + c * STAGE_COL_BYTES + piece * 16);
+        const u32x2 up = *reinterpret_cast<const u32x2*>(region + c * STAGE_COL_BYTES + piece * 16 + 8);
+        const u32x4 v = {lo[0], lo[1], up[0], up[1]};
+        *reinterpret_cast<u32x4*>(ct + (size_t)(colw + 32 * h + c) * p.ct_rows + piece * 8) = v;
+      }
+    }
+  }
+}
+
+template <int EPI, int PRIO>
+__global__ __launch_bounds__(NW * 64) void gemm_bf16_x32(HGemmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) u16 smem_x[];
+  const unsigned lds_base = (unsigned)(size_t)((__attribute__((address_space(3))) const void*)smem_x);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, kg = lane >> 4;
+  const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
+
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  // tile loads: a wave-uniform base per operand, advanced with scalar adds, plus one constant byte
+  // offset per lane and instruction (no vector arithmetic in the K loop)
+  const int lrow = lane / VPR, pc = lane % VPR;
+  unsigned offa[NIA], offb[NIB];
+#pragma unroll
+  for (int j = 0; j < NIA; ++j) {
+    const int row = (j * NW + wave) * RPI + lrow;
+    offa[j] = 2u * ((unsigned)row * (unsigned)p.lda + (unsigned)(pc ^ swz_a(row)) * 8u);
+  }
+#pragma unroll
+  for (int j = 0; j < NIB; ++j) {
+    const int row = (j * NW + wave) * RPI + lrow;
+    offb[j] = 2u * ((unsigned)row * (unsigned)p.ldb + (unsigned)(pc ^ swz_b(row)) * 8u);
+  }
+  const u16* a_base = p.A + (size_t)blockIdx.z * p.batchA + (size_t)m0 * p.lda;
+  const u16* b_base = p.B + (size_t)blockIdx.z * p.batchB + (size_t)n0 * p.ldb;
+  auto issue_a = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < NIA; ++j)
+      load_to_lds(a_base, offa[j], lds_base + 2u * (unsigned)(buf * A_ELEMS + (j * NW + wave) * RPI * BK));
+    a_base += BK;
+  };
+  auto issue_b = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < NIB; ++j)
+      load_to_lds(b_base, offb[j], lds_base + 2u * (unsigned)(2 * A_ELEMS + buf * B_ELEMS + (j * NW + wave) * RPI * BK));
+    b_base += BK;
+  };
+
+  // LDS byte addresses of this lane's fragments for K chunk 0 / 1 (block 0, buffer 0); blocks and
+  // buffers are immediate offsets.  The empty asm keeps the compiler from re-deriving them in the loop.
+  unsigned q_addr[2], p_addr[2];
+#pragma unroll
+  for (int kc = 0; kc < 2; ++kc) {
+    const int ra = wm0 + l16, rb = wn0 + 8 * (l16 >> 2) + (l16 & 3);
+    q_addr[kc] = lds_base + 2u * (unsigned)(ra * BK + ((kc * 4 + kg) ^ swz_a(ra)) * 8);
+    p_addr[kc] = lds_base + 2u * (unsigned)(2 * A_ELEMS + rb * BK + ((kc * 4 + kg) ^ swz_b(rb)) * 8);
+    asm volatile("" : "+v"(q_addr[kc]), "+v"(p_addr[kc]));
+  }
+  auto load_q = [&](bf16x8 (&f)[4], int buf, int kc, int half) __attribute__((always_inline)) {
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj)
+      f[jj] = *reinterpret_cast<lds_frag*>((__attribute__((address_space(3))) const char*)(size_t)(
+          q_addr[kc] + 2u * (unsigned)(buf * A_ELEMS + (half * 4 + jj) * 16 * BK)));
+  };
+  auto load_p = [&](bf16x8 (&f)[PB], int buf, int kc) __attribute__((always_inline)) {
+#pragma unroll
+    for (int ip = 0; ip < PB; ++ip)
+      f[ip] = *reinterpret_cast<lds_frag*>((__attribute__((address_space(3))) const char*)(size_t)(
+          p_addr[kc] + 2u * (unsigned)(buf * B_ELEMS + (32 * (ip >> 1) + 4 * (ip & 1)) * BK)));
+  };
+
+  f32x4 acc[QB][PB];
+#pragma unroll
+  for (int jq = 0; jq < QB; ++jq)
+#pragma unroll
+    for (int ip = 0; ip < PB; ++ip)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[jq][ip][r] = 0.0f;
+
+  const int nk = p.K / BK;
+  bf16x8 fq[2][4], fp[2][PB];
+  // sub-chunk s of a step: K chunk s / 2, m blocks 4 (s % 2) .. 4 (s % 2) + 3
+  auto multiply = [&](int s) __attribute__((always_inline)) {
+    if (PRIO == 1) __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+      for (int ip = 0; ip < PB; ++ip)
+        acc[(s & 1) * 4 + jj][ip] =
+            __builtin_amdgcn_mfma_f32_16x16x32_bf16(fp[(s >> 1) & 1][ip], fq[s & 1][jj], acc[(s & 1) * 4 + jj][ip], 0, 0, 0);
+    if (PRIO == 1) __builtin_amdgcn_s_setprio(0);
+  };
+
+  if (nk > 0) {
+    issue_a(0);
+    issue_b(0);
+  }
+  if (nk > 1) {
+    issue_a(1);
+    issue_b(1);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(INSTR));
+  } else {
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+  }
+  ring_barrier();
+  load_q(fq[0], 0, 0, 0);
+  load_p(fp[0], 0, 0);
+  // Step t multiplies buffer t % 2.  Before its last sub-chunk every wavefront has issued all its
+  // reads of that buffer; it waits for them and for tile t+1 (the other buffer), then the barrier,
+  // then tile t+2 is requested into the buffer just read out.  The first fragments of tile t+1 are
+  // fetched under the last sub-chunk's MFMAs.
+  auto step = [&](int t, auto cur_c, auto steady_c) __attribute__((always_inline)) {
+    constexpr int cur = decltype(cur_c)::value;
+    constexpr bool steady = decltype(steady_c)::value;  // tile t+2 exists
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int ns = s + 1;
+      if (ns < 4) {
+        load_q(fq[ns & 1], cur, ns >> 1, ns & 1);
+        if ((ns & 1) == 0) load_p(fp[(ns >> 1) & 1], cur, ns >> 1);
+      } else {  // after the last tile: a harmless read of ring memory, keeps one code path
+        load_q(fq[0], cur ^ 1, 0, 0);
+        load_p(fp[0], cur ^ 1, 0);
+      }
+      if (s == 2) __builtin_amdgcn_sched_barrier(0);  // the last reads of this buffer go out before these MFMAs
+      multiply(s);
+      if (s == 2) {
+        __builtin_amdgcn_sched_barrier(0);  // and the MFMAs stay above the barrier
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0) & 0xc07f);  // vmcnt(0) and lgkmcnt(0)
+        ring_barrier();
+        if (steady || t + 2 < nk) issue_a(cur);
+      }
+      if (s == 3) {
+        if (steady || t + 2 < nk) issue_b(cur);
+      }
+    }
+  };
+  int t = 0;
+  for (; t + 4 <= nk; t += 2) {
+    step(t, std::integral_constant<int, 0>{}, std::true_type{});
+    step(t + 1, std::integral_constant<int, 1>{}, std::true_type{});
+  }
+  static_for_h<3>([&](auto sc) {
+    constexpr int s = decltype(sc)::value;
+    if (t + s < nk) step(t + s, std::integral_constant<int, s % 2>{}, std::false_type{});
+  });
+
+  unsigned char* region = nullptr;
+  if (EPI != EPH_F32 && p.Ct) {
+    __syncthreads();  // every wavefront is done with the operand tiles: the LDS is free for the staging
+    region = reinterpret_cast<unsigned char*>(smem_x) + (size_t)wave * STAGE_REGION;
+  }
+  store_x32<EPI>(p, acc, m0 + wm0, n0 + wn0, lane, region);
+}
+
+template <int EPI, int PRIO>
+hipError_t launch_one(HGemmArgs& p, int batch, hipStream_t s) {
+  auto kern = gemm_bf16_x32<EPI, PRIO>;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), LDS_BYTES); e != hipSuccess) return e;
+  p.tiles_m = p.M / BM;
+  p.tiles_n = p.N / BN;
+  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(NW * 64), LDS_BYTES, s, p);
+  return hipGetLastError();
+}
+
+template <int PRIO>
+hipError_t launch_prio(HGemmArgs& p, int batch, int epi, hipStream_t s) {
+  switch (epi) {
+    case EPH_F32: return launch_one<EPH_F32, PRIO>(p, batch, s);
+    case EPH_BIAS_RELU: return launch_one<EPH_BIAS_RELU, PRIO>(p, batch, s);
+    case EPH_MASK: return launch_one<EPH_MASK, PRIO>(p, batch, s);
+    default: return launch_one<EPH_BF16, PRIO>(p, batch, s);
+  }
+}
+
+}  // namespace
+
+hipError_t launch_x32(HGemmArgs& p, int batch, int epi, bool prio, hipStream_t s) {
+  return prio ? launch_prio<1>(p, batch, epi, s) : launch_prio<0>(p, batch, epi, s);
+}
+
+}  // namespace mi
