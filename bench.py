@@ -175,6 +175,8 @@ def main():
     mfma_only = {"unit": "TFLOP/s", "random_operands": mfma_rate(2), "ones": mfma_rate(1), "zeros": mfma_rate(0),
                  "how": "loop of independent MFMAs on register operands, no memory traffic, measured right "
                         "after the steps above (mi_probe_mfma_rate)"}
+    if dtype == "bf16":  # the large GEMMs use 16x16x32 MFMAs (the figures above); the 32x32x16 shape for comparison
+        mfma_only["random_operands_32x32x16"] = mfma_rate(3)
 
     rows = R * B
     # FLOP of the forward / weight-gradient / input-gradient GEMM of layer l: 2 * rows * N_l * N_{l+1}.

@@ -190,9 +190,11 @@ int mi_set_hgemm_variant(int variant);
 /*
  * Measurement aid without a counterpart in the reference: the rate, in TFLOP/s, of a loop of
  * independent MFMAs on register operands (v_mfma_f32_32x32x2_f32 for MI_F32,
- * v_mfma_f32_32x32x16_bf16 for MI_BF16) with no memory traffic, i.e. what the matrix cores of
- * this device sustain at best.  operands: 0 = zeros, 1 = ones, 2 = pseudo-random values in
- * [-1, 1) -- the bf16 rate is power-limited and depends on them.  Blocks until the measurement is
+ * v_mfma_f32_16x16x32_bf16, the instruction of the large bf16 GEMMs, for MI_BF16) with no memory
+ * traffic, i.e. what the matrix cores of this device sustain at best.  operands: 0 = zeros,
+ * 1 = ones, 2 = pseudo-random values in [-1, 1) -- the bf16 rate is power-limited and depends on
+ * them -- 3 = the same random values through v_mfma_f32_32x32x16_bf16 (MI_BF16; for fp32 the same
+ * as 2), which sustains less on this device.  Blocks until the measurement is
  * done (about 0.4 s; the rate is the average over the second half, so that idle clocks do not
  * enter); allocates and frees a small device buffer.
  */

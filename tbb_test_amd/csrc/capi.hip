@@ -870,7 +870,7 @@ int mi_set_hgemm_variant(int variant) {
 
 int mi_probe_mfma_rate(int dtype, int operands, double* tflops, void* stream) {
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "dtype must be MI_F32 or MI_BF16 (got %d)", dtype);
-  MI_REQUIRE(operands >= 0 && operands <= 2, "operands must be 0 (zeros), 1 (ones) or 2 (random), got %d", operands);
+  MI_REQUIRE(operands >= 0 && operands <= 3, "operands must be 0 (zeros), 1 (ones), 2 (random) or 3 (random, 32x32x16 bf16 MFMAs), got %d", operands);
   MI_REQUIRE(tflops != nullptr, "null result pointer");
   hipError_t e = mi::probe_mfma_rate(dtype == MI_BF16, operands, tflops, as_stream(stream));
   if (e != hipSuccess) return hip_fail(e, "mi_probe_mfma_rate");

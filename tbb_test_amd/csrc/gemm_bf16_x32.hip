@@ -75,12 +75,28 @@ __device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][P
   } else {
     u16* __restrict__ ch = reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC;
     u32x4 pk[QB][2];  // the rounded results: eight consecutive columns per register quadruple
+    // The whole mask of the wavefront's tile is requested before the first result is stored: the
+    // counter that a load is waited for with retires loads and stores in order, so a mask load
+    // issued after a store would wait for that store to reach the L2 first, sixteen times in a row.
+    u32x4 mk_all[QB][2];
+    if (EPI == EPH_MASK) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int jq = 0; jq < QB; ++jq)
+          mk_all[jq][h] = *reinterpret_cast<const u32x4*>(p.mask + (size_t)(row0 + 16 * jq + l16) * p.ldmask + colw + 32 * h + 8 * q);
+    }
+    float bias_all[2][8];  // likewise the bias of the lane's sixteen columns
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        bias_all[h][e] = (EPI == EPH_BIAS_RELU && p.bias) ? p.bias[colw + 32 * h + 8 * q + e] : 0.0f;
+    asm volatile("" ::: "memory");  // the stores below stay below
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int col = colw + 32 * h + 8 * q;
-      float bias_v[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) bias_v[e] = (EPI == EPH_BIAS_RELU && p.bias) ? p.bias[col + e] : 0.0f;
+      const float(&bias_v)[8] = bias_all[h];
 #pragma unroll
       for (int jq = 0; jq < QB; ++jq) {
         const int row = row0 + 16 * jq + l16;
@@ -94,7 +110,7 @@ __device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][P
             if (p.relu) v[e] = v[e] > 0.0f ? v[e] : 0.0f;
           }
         } else if (EPI == EPH_MASK) {
-          const u32x4 mk = *reinterpret_cast<const u32x4*>(p.mask + (size_t)row * p.ldmask + col);
+          const u32x4 mk = mk_all[jq][h];
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const u16 m = (u16)(mk[e >> 1] >> (16 * (e & 1)));
