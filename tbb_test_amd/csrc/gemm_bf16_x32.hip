@@ -19,7 +19,8 @@
 // (columns 8q .. 8q+7 and 32 + 8q .. 32 + 8q+7 of the wavefront's 64, q = lane / 16):
 //   block ip, register-side index 4q + r  ->  column 32 * (ip / 2) + 8q + 4 * (ip % 2) + r.
 // The epilogue therefore writes C, and reads the ReLU mask, in 16-byte pieces per lane with no
-// shuffling (fp32 results: 32 contiguous bytes per lane).  The B tile's LDS swizzle is chosen for
+// shuffling.  (The fp32 instance keeps the natural row order instead: there a block's four
+// registers are 16 contiguous bytes already.)  The B tile's LDS swizzle is chosen for
 // that row order: the 16 lanes of a quarter-wave read rows 8q' + r' (+ multiples of 4 and 32),
 // swizzle = 2 * ((row / 8) % 4) + (row / 2) % 2 gives them 16 distinct 16-byte slots.
 //
@@ -64,12 +65,9 @@ __device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][P
     float* __restrict__ cf = reinterpret_cast<float*>(p.C) + (size_t)blockIdx.z * p.batchC;
 #pragma unroll
     for (int jq = 0; jq < QB; ++jq) {
-      float* dst = cf + (size_t)(row0 + 16 * jq + l16) * p.ldc + colw + 8 * q;
+      float* dst = cf + (size_t)(row0 + 16 * jq + l16) * p.ldc + colw + 4 * q;  // natural B order, see the kernel
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        *reinterpret_cast<f32x4*>(dst + 32 * h) = acc[jq][2 * h];
-        *reinterpret_cast<f32x4*>(dst + 32 * h + 4) = acc[jq][2 * h + 1];
-      }
+      for (int ip = 0; ip < PB; ++ip) *reinterpret_cast<f32x4*>(dst + 16 * ip) = acc[jq][ip];
     }
     return;
   } else {
@@ -190,6 +188,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_x32(HGemmArgs p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l16 = lane & 15, kg = lane >> 4;
+  // fp32 results: a lane's four registers of a block are 16 contiguous bytes, so the rows of the B
+  // tile keep their natural order (block ip = columns 16 ip .. 16 ip + 15, lane quarter q columns
+  // 4q .. 4q+3 of them) and a store instruction writes 64 contiguous bytes per row; the dealt order
+  // described at the top would leave 16-byte holes that the next instruction fills.
+  constexpr bool NAT = EPI == EPH_F32;
   const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
 
   int tile_m, tile_n;
@@ -208,7 +211,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_x32(HGemmArgs p) {
 #pragma unroll
   for (int j = 0; j < NIB; ++j) {
     const int row = (j * NW + wave) * RPI + lrow;
-    offb[j] = 2u * ((unsigned)row * (unsigned)p.ldb + (unsigned)(pc ^ swz_b(row)) * 8u);
+    offb[j] = 2u * ((unsigned)row * (unsigned)p.ldb + (unsigned)(pc ^ (NAT ? swz_a(row) : swz_b(row))) * 8u);
   }
   const u16* a_base = p.A + (size_t)blockIdx.z * p.batchA + (size_t)m0 * p.lda;
   const u16* b_base = p.B + (size_t)blockIdx.z * p.batchB + (size_t)n0 * p.ldb;
@@ -230,9 +233,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_x32(HGemmArgs p) {
   unsigned q_addr[2], p_addr[2];
 #pragma unroll
   for (int kc = 0; kc < 2; ++kc) {
-    const int ra = wm0 + l16, rb = wn0 + 8 * (l16 >> 2) + (l16 & 3);
+    const int ra = wm0 + l16, rb = NAT ? wn0 + l16 : wn0 + 8 * (l16 >> 2) + (l16 & 3);
     q_addr[kc] = lds_base + 2u * (unsigned)(ra * BK + ((kc * 4 + kg) ^ swz_a(ra)) * 8);
-    p_addr[kc] = lds_base + 2u * (unsigned)(2 * A_ELEMS + rb * BK + ((kc * 4 + kg) ^ swz_b(rb)) * 8);
+    p_addr[kc] = lds_base + 2u * (unsigned)(2 * A_ELEMS + rb * BK + ((kc * 4 + kg) ^ (NAT ? swz_a(rb) : swz_b(rb))) * 8);
     asm volatile("" : "+v"(q_addr[kc]), "+v"(p_addr[kc]));
   }
   auto load_q = [&](bf16x8 (&f)[4], int buf, int kc, int half) __attribute__((always_inline)) {
@@ -245,7 +248,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_x32(HGemmArgs p) {
 #pragma unroll
     for (int ip = 0; ip < PB; ++ip)
       f[ip] = *reinterpret_cast<lds_frag*>((__attribute__((address_space(3))) const char*)(size_t)(
-          p_addr[kc] + 2u * (unsigned)(buf * B_ELEMS + (32 * (ip >> 1) + 4 * (ip & 1)) * BK)));
+          p_addr[kc] + 2u * (unsigned)(buf * B_ELEMS + (NAT ? 16 * ip : 32 * (ip >> 1) + 4 * (ip & 1)) * BK)));
   };
 
   f32x4 acc[QB][PB];
