@@ -86,6 +86,52 @@ def cpu_baseline(nf, B, R, lr, budget_s):
     return port.run(nf, B, R, lr, budget_s)
 
 
+def raw_gemm(args, np, capi):
+    """One GEMM entry point alone, as the profiles quote it: C = A[M,K] * B[N,K]^T (+ ReLU), operands with
+    random signs, exponents and mantissas (what the power-limited bf16 rate depends on), K launches between
+    two stream synchronisations."""
+    import ctypes
+    import time
+
+    M, N, K = (int(x) for x in args.gemm.split(","))
+    lib = capi.lib()
+    if args.hvariant:
+        capi.check(lib.mi_set_hgemm_variant(args.hvariant))
+    if args.variants:
+        for kind, v in enumerate(int(x) for x in args.variants.split(",")):
+            capi.check(lib.mi_set_gemm_variant(kind, v))
+    rng = np.random.default_rng(args.seed)
+    bf16 = args.gemm_dtype == "bf16"
+
+    def operand(rows):
+        if bf16:  # sign | exponent 2^-3 .. 2^2 | 7 mantissa bits
+            v = (rng.integers(0, 2, (rows, K), dtype=np.uint16) << 15) | ((0x7c + rng.integers(0, 6, (rows, K), dtype=np.uint16)) << 7) \
+                | rng.integers(0, 128, (rows, K), dtype=np.uint16)
+            return capi.DeviceBuffer.from_numpy(v.astype(np.uint16))
+        return capi.DeviceBuffer.from_numpy(rng.standard_normal((rows, K), dtype=np.float32))
+
+    A, Bm = operand(M), operand(N)
+    C = capi.DeviceBuffer(M * N * (2 if bf16 else 4))
+    fn = lib.mi_hgemm_nt if bf16 else lib.mi_sgemm_nt
+
+    def launch():
+        capi.check(fn(M, N, K, A.ptr, K, Bm.ptr, K, C.ptr, N, None, 1, None))
+
+    for _ in range(max(args.warmup, 20)):   # also brings the clocks up
+        launch()
+    capi.check(lib.mi_stream_sync(None))
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        launch()
+    capi.check(lib.mi_stream_sync(None))
+    us = (time.perf_counter() - t0) / args.steps * 1e6
+    peak = 2516.6 if bf16 else 157.3
+    tflops = 2.0 * M * N * K / us / 1e6
+    print(json.dumps({"gemm": f"{args.gemm_dtype} nt {M}x{N}x{K}", "hvariant": args.hvariant, "variants": args.variants,
+                      "launches": args.steps, "us_per_launch": round(us, 1), "tflops": round(tflops, 1),
+                      "frac_of_peak": round(tflops / peak, 4)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -100,6 +146,10 @@ def main():
     ap.add_argument("--variants", default="", help="tuning: forced GEMM tile variants 'nt,nn,tn'")
     ap.add_argument("--serial-backward", action="store_true", help="whole backward pass on one stream")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--gemm", default="", metavar="M,N,K",
+                    help="instead of the training step: time the forward-type GEMM entry point alone (mi_hgemm_nt / "
+                         "mi_sgemm_nt, dtype of --gemm-dtype, dense random operands) and print one JSON line")
+    ap.add_argument("--gemm-dtype", default="bf16", choices=["bf16", "f32"])
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -110,6 +160,10 @@ def main():
     import numpy as np
 
     from tbb_test_amd import capi, hostlib
+
+    if args.gemm:
+        raw_gemm(args, np, capi)
+        return
 
     nf, B, R, dtype = CONFIGS[args.config]
     layers = len(nf) - 1
@@ -230,8 +284,9 @@ def main():
         "reduce_gbps": round(upd_gbps, 1),
         "weights_finite": finite,
         "roofline": {"kernel": "gemm_f32_dma (nt, nn, tn)" if dtype == "f32" else
-                               "gemm_bf16_dma (spans of the weight gradient include its row-sum kernel and, for "
-                               "operands no GEMM epilogue wrote transposed, the transpose launches)",
+                               "gemm_bf16_x32 (spans of the weight gradient include the column-sum fold or row-sum "
+                               "kernel of the bias gradient and, for operands no GEMM epilogue wrote transposed, the "
+                               "transpose launches)",
                      "bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(gemm_tflops / peak, 4),
                      "traffic": traffic.get("gemm"), "traffic_note": traffic_note,

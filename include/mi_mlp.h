@@ -159,7 +159,7 @@ int mi_reduce_sgd_bf16t_raw(float* W, void* W_bf16, void* Wt_bf16, const float* 
 
 /*
  * bf16 variants of the three GEMMs (bf16 stored as 16-bit words, fp32 accumulation on
- * v_mfma_f32_32x32x16_bf16).  A bf16 MFMA reads 8 consecutive k per lane, so every operand must be
+ * v_mfma_f32_16x16x32_bf16 for the large shapes, v_mfma_f32_32x32x16_bf16 otherwise).  A bf16 MFMA reads 8 consecutive k per lane, so every operand must be
  * K-contiguous; where the fp32 call site reads a row-contiguous operand, the bf16 entry point
  * takes its transposed copy (mi_transpose_bf16 makes one):
  *   mi_hgemm_nt  forward          C[M x N] (bf16) = A[M x K] * B[N x K]^T + bias, optional ReLU
