@@ -129,6 +129,7 @@ __device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][P
       // Column sums of the rounded values over the wavefront's 128 rows: a lane adds its eight rows
       // in block order, the 16 lanes of a quarter-wave are folded with a fixed butterfly.
       float* part = p.colsum_part + (size_t)(row0 / WTM) * p.N;
+      float tot[2][8];
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -141,8 +142,18 @@ __device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][P
           }
 #pragma unroll
           for (int off = 1; off < 16; off <<= 1) c += __shfl_xor(c, off, 64);
-          if (l16 == 0) part[colw + 32 * h + 8 * q + e] = c;
+          tot[h][e] = c;
         }
+      // one lane of each quarter-wave writes its two runs of eight sums as 16-byte pieces (single
+      // floats, a store instruction apart, reached the memory as one 64-byte write each)
+      if (l16 == 0) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          float* dst = part + colw + 32 * h + 8 * q;
+          *reinterpret_cast<f32x4*>(dst) = f32x4{tot[h][0], tot[h][1], tot[h][2], tot[h][3]};
+          *reinterpret_cast<f32x4*>(dst + 4) = f32x4{tot[h][4], tot[h][5], tot[h][6], tot[h][7]};
+        }
+      }
     }
     if (!p.Ct) return;
     // Transposed copy: the tile lies inside one row group (ct_rows is a multiple of the tile height).

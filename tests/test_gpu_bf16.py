@@ -112,6 +112,45 @@ def test_hgemm_on_operands_that_allow_no_vector_access(shape):
     assert np.all(out[:, N:] == 0)   # nothing written between the rows of C
 
 
+@pytest.mark.parametrize("variant", [0, 27])
+@pytest.mark.parametrize("ldc_extra,c_shift", [(4, 0), (0, 1), (8, 0)])
+def test_hgemm_16x16x32_kernel_gives_way_when_c_or_the_mask_allow_no_16_byte_access(variant, ldc_extra, c_shift):
+    """The 16x16x32 kernel writes C and reads the ReLU mask in 16-byte pieces.  With a leading
+    dimension of C that is no multiple of 8, or C (or the mask) starting off a 16-byte boundary, the
+    32x32x16 kernel of the same tile runs instead: results as good, nothing written between rows.
+    (ldc_extra = 8 keeps the alignment: the 16x16x32 kernel itself with a padded C.)"""
+    M, N, K = 512, 256, 128
+    rng = np.random.default_rng(ldc_extra * 7 + c_shift)
+    A = bf16_round(rng.uniform(-1, 1, (M, K)))
+    B = bf16_round(rng.uniform(-1, 1, (N, K)))
+    bias = rng.uniform(-1, 1, N).astype(np.float32)
+    act = bf16_round(np.maximum(rng.uniform(-1, 1, (M, N)), 0))
+    ldc = N + ldc_extra
+    lib = capi.lib()
+    dA, dB, dbias = dev16(A), dev16(B), capi.DeviceBuffer.from_numpy(bias)
+    mask_padded = np.zeros((M, ldc), np.uint16)
+    mask_padded[:, :N] = to_bf16_bits(act)
+    dmask = capi.DeviceBuffer.from_numpy(np.concatenate([np.zeros(c_shift, np.uint16), mask_padded.ravel()]))
+    dC = capi.DeviceBuffer((c_shift + M * ldc) * 2)
+    capi.check(lib.mi_set_hgemm_variant(variant))
+    try:
+        for kind in ("forward", "input gradient"):
+            dC.zero()
+            if kind == "forward":
+                capi.check(lib.mi_hgemm_nt(M, N, K, dA.ptr, K, dB.ptr, K, dC.ptr + 2 * c_shift, ldc, dbias.ptr, 1, None))
+                want = oracle.fc_forward(A, B, bias, True)
+            else:
+                capi.check(lib.mi_hgemm_nn(M, N, K, dA.ptr, K, dB.ptr, K, dC.ptr + 2 * c_shift, ldc,
+                                           dmask.ptr + 2 * c_shift, ldc, None))
+                want = oracle.fc_dgrad(A, np.ascontiguousarray(B.T), act)
+            capi.check(lib.mi_stream_sync(None))
+            out = from_bf16_bits(dC.to_numpy((c_shift + M * ldc,), np.uint16))[c_shift:].reshape(M, ldc)
+            assert rel_err(out[:, :N], want) <= 4e-3, kind
+            assert np.all(out[:, N:] == 0), kind
+    finally:
+        lib.mi_set_hgemm_variant(0)
+
+
 @pytest.mark.parametrize("variant", HVARIANTS)
 @pytest.mark.parametrize("R", [1, 3])
 @pytest.mark.parametrize("shape", HSHAPES)
