@@ -205,6 +205,13 @@ def main():
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
 
+    # the weight restore alone (it is inside every timed step above, see the module docstring)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        h.restore_weights()
+    h.sync()
+    restore_ms = (time.perf_counter() - t0) / args.steps * 1e3
+
     # per-kernel durations: same loop again with a HIP event pair around every launch
     h.enable_timing(True)
     h.reset_timings()
@@ -280,6 +287,7 @@ def main():
                    "schedule": schedule, "device": info["name"], "num_cus": info["num_cus"]},
         "gemm_flop_per_step": gemm_flop_step,
         "phase_ms_per_step": {k: round(v, 4) for k, v in per_phase.items()},
+        "restore_ms_per_step": round(restore_ms, 4),   # part of ms_per_step, not of the reference's step
         "gemm_tflops": round(gemm_tflops, 2),
         "reduce_gbps": round(upd_gbps, 1),
         "weights_finite": finite,
