@@ -13,11 +13,13 @@
 //   weight gradient  dW_r = dZ_r^T * A_r         A = dZ_r^T,  B = A_r^T      (reference call sites
 //                                                mlp_omp.cc:474-488, 657-671, 565-580)
 //
-// Two kernels.  gemm_bf16_mfma stages the tile through registers: three LDS buffers, tile t+1
+// Two kernels here.  gemm_bf16_mfma stages the tile through registers: three LDS buffers, tile t+1
 // written to LDS at the top of step t, loads of tile t+2 issued right after, one LDS-only barrier
 // in the middle of the step, operand fragments of the next 16-wide K chunk fetched while the
-// current chunk is multiplied.  gemm_bf16_dma (further down; the kernel of the large GEMMs) loads
-// global -> LDS directly.
+// current chunk is multiplied.  gemm_bf16_dma (further down) loads global -> LDS directly.  The
+// large GEMMs (256 x 256 tiles covering the CUs, K a multiple of 64) run on a third kernel built
+// on v_mfma_f32_16x16x32_bf16, gemm_bf16_x32.hip, which the dispatch below selects; gemm_bf16_dma
+// stays for the BK = 32 ring, for outputs that allow no 16-byte stores, and for comparison.
 // Tiles are stored [row][BK] with the 16-byte chunks of a row XOR-swizzled (no padding, no bank
 // conflicts); a lane fetches its 8 k values of one 32 x 32 block with one 16-byte LDS read.
 #include <hip/hip_runtime.h>
