@@ -92,12 +92,12 @@ __device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][P
         bias_all[h][e] = (EPI == EPH_BIAS_RELU && p.bias) ? p.bias[colw + 32 * h + 8 * q + e] : 0.0f;
     asm volatile("" ::: "memory");  // the stores below stay below
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int col = colw + 32 * h + 8 * q;
-      const float(&bias_v)[8] = bias_all[h];
+    for (int jq = 0; jq < QB; ++jq) {
+      const int row = row0 + 16 * jq + l16;
 #pragma unroll
-      for (int jq = 0; jq < QB; ++jq) {
-        const int row = row0 + 16 * jq + l16;
+      for (int h = 0; h < 2; ++h) {  // both halves of a row's 128-byte line back to back
+        const int col = colw + 32 * h + 8 * q;
+        const float(&bias_v)[8] = bias_all[h];
         float v[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = acc[jq][2 * h + (e >> 2)][e & 3];
