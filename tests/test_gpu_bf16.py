@@ -55,7 +55,9 @@ HSHAPES = [(64, 64, 32), (128, 128, 64), (256, 256, 96), (512, 256, 128), (256, 
            (129, 64, 40), (256, 256, 512),
            # K loops of the direct-load kernels: one step, and every length of the conditional tail after
            # the branch-free turns of the ring (two buffers at BK = 64, four at BK = 32)
-           (256, 256, 64), (256, 256, 192), (256, 256, 320), (256, 256, 448)]
+           (256, 256, 64), (256, 256, 192), (256, 256, 320), (256, 256, 448),
+           # twelve 256 x 256 tiles, three K steps
+           (1024, 768, 192)]
 HVARIANTS = [0, 3, 4, 5, 13, 17, 19, 21, 22, 25, 27, 28]   # 21, 22: guarded any-shape MFMA instances; 25: 19 without wave priorities; 27, 28: 16x16x32 MFMAs
 
 
