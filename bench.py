@@ -7,9 +7,10 @@ A "step" is one pass of the whole hot path over one batch of seeded synthetic in
 GEMMs, L weight-gradient GEMMs (R replicas each), L bias gradients, L input-gradient GEMMs and
 the R-way gradient reduce with the SGD update.  Inputs and weights are resident in HBM before
 the timed region starts.  Default schedule: the weight-gradient GEMMs and the per-layer reduce+SGD
-launches trail the chain of input-gradient GEMMs on a second stream.  Every timed step starts from the initial weights (a device-to-device
-restore that is inside the timed region), so that values stay finite however many sum-reduced
-SGD steps are run.
+launches trail the chain of input-gradient GEMMs on a second stream.  The timed loop is the
+reference's: K consecutive steps, each on the weights the step before left, with the reference's
+learning rate of 1e-10 (mlp_omp.cc:435-737 with alpha at :609,699,718,729), at which the
+sum-reduced updates stay finite however many steps are run.
 
 Prints one JSON line:
   value          whole-step throughput, TFLOP/s on the reference's FLOP model
@@ -65,7 +66,7 @@ def kernel_source_hash():
 
 def measured_traffic(config):
     """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
-    scaled by what the same counter reads for the plain device copy of the weight restore), as
+    scaled by what the same counter reads for the plain device copy of the weight snapshot), as
     recorded in profiles/traffic_pmc.json together with the hash of the kernel sources they were
     measured on.  Returns ({"gemm": bytes, "reduce": bytes}, note); figures are None when nothing
     was recorded for the configuration or when the kernels have changed since."""
@@ -138,7 +139,7 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
-    ap.add_argument("--lr", type=float, default=0.01)
+    ap.add_argument("--lr", type=float, default=1e-10, help="learning rate (default: the reference benchmark's alpha)")
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--flat-update", action="store_true",
                     help="one update launch at the end of the step instead of per-layer updates on the second stream")
@@ -185,7 +186,6 @@ def main():
     params, _ = h.param_count()
 
     def one_step():
-        h.restore_weights()
         h.step(args.lr)
 
     # Untimed spin-up so that the GPU has left its idle clock state before anything is measured
@@ -205,14 +205,9 @@ def main():
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
 
-    # the weight restore alone (it is inside every timed step above, see the module docstring)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        h.restore_weights()
-    h.sync()
-    restore_ms = (time.perf_counter() - t0) / args.steps * 1e3
-
-    # per-kernel durations: same loop again with a HIP event pair around every launch
+    # per-kernel durations: K more steps, from the initial weights again, with a HIP event pair
+    # around every launch
+    h.restore_weights()
     h.enable_timing(True)
     h.reset_timings()
     for _ in range(args.steps):
@@ -287,7 +282,6 @@ def main():
                    "schedule": schedule, "device": info["name"], "num_cus": info["num_cus"]},
         "gemm_flop_per_step": gemm_flop_step,
         "phase_ms_per_step": {k: round(v, 4) for k, v in per_phase.items()},
-        "restore_ms_per_step": round(restore_ms, 4),   # part of ms_per_step, not of the reference's step
         "gemm_tflops": round(gemm_tflops, 2),
         "reduce_gbps": round(upd_gbps, 1),
         "weights_finite": finite,

@@ -1,8 +1,11 @@
 """GPU parity of exactly what bench.py times: a handle built with MI_FLAG_PER_LAYER_UPDATE (graph
-on), snapshot, then [restore, step] repeated so that the step replays its captured graph with the
-weight-gradient GEMMs and the per-layer reduce + SGD launches trailing the input-gradient chain on
-the second stream -- the GPU counterpart of the reference loop with OVERLAP_ALL_REDUCE
-(mlp_omp.cc:435-737 with :601-615,692-723).
+on) whose step replays its captured graph with the weight-gradient GEMMs and the per-layer
+reduce + SGD launches trailing the input-gradient chain on the second stream -- the GPU
+counterpart of the reference loop with OVERLAP_ALL_REDUCE (mlp_omp.cc:435-737 with
+:601-615,692-723).  Two loops: consecutive steps (bench.py's and the reference's loop, each step on
+the weights the step before left), and snapshot, then [restore, step] repeated (every replay
+starts from the same weights, so one oracle step checks a replayed step at a learning rate that
+moves the weights visibly).
 
 Config 2 (the benchmark's headline) runs at full size against the float64-accumulating oracle and,
 bit for bit, against the serial eager schedule.  Config 5 (bf16, 52.8 TFLOP per step) is checked
@@ -32,7 +35,7 @@ def build(nf, B, R, seed, dtype=capi.MI_F32, flags=0):
 
 
 def bench_loop(h, steps, snapshot=True):
-    """The loop of bench.py: every step starts from the snapshot."""
+    """Every step starts from the snapshot (a benchmark loop whose values cannot drift)."""
     if snapshot:
         h.snapshot_weights()
     for _ in range(steps):
@@ -93,6 +96,54 @@ def test_config_2_benchmarked_schedule_full_size():
             assert np.array_equal(bits(h.wgrad_of(l, r)), bits(hs.wgrad_of(l, r))), f"dW {l} {r}"
     h.close()
     hs.close()
+
+
+@pytest.mark.parametrize("lr", [1e-10, 1e-5])
+def test_config_2_consecutive_steps_as_the_benchmark_runs_them(lr):
+    """bench.py's timed loop at full size: consecutive steps, no restore in between, at the
+    reference's alpha (1e-10, mlp_omp.cc:609: an update of about one ulp of a weight) and at a rate
+    that moves the weights by some tenths of a per cent per step.  Step 1 runs eagerly, steps 2 and 3
+    replay the graph.  Bit for bit what the serial eager schedule computes.  At the larger rate the
+    third step is also checked against the oracle started from the device's weights after two steps:
+    a free-running oracle chain cannot be held to 1e-4 here, because a ReLU mask entry that
+    rounding decides differently (14 of 37 million in the first step) changes a whole row of every
+    earlier layer's gradient by per cents, and the next steps amplify it (9 000 entries two steps
+    later)."""
+    nf, B, R = [1024] * 9, 1024, 4
+    L = len(nf) - 1
+    h, X, Ws, dY = build(nf, B, R, seed=1, flags=BENCH_FLAGS)
+    hs, *_ = build(nf, B, R, seed=1, flags=capi.FLAG_NO_GRAPH | capi.FLAG_SERIAL_BACKWARD)
+    for step in range(3):
+        if step == 2:
+            h.sync()
+            W2 = [h.weight(l) for l in range(L)]
+            b2 = [h.bias(l) for l in range(L)]
+        h.step(lr)
+        hs.step(lr)
+    h.sync(); hs.sync()
+    assert h.schedule()["graph"] and h.schedule()["dual_streams"] and h.schedule()["per_layer_update"]
+    assert not hs.schedule()["graph"] and not hs.schedule()["dual_streams"]
+    assert np.array_equal(bits(h.dx()), bits(hs.dx()))
+    for l in range(L):
+        assert np.array_equal(bits(h.weight(l)), bits(hs.weight(l))), f"W {l}"
+        assert np.array_equal(bits(h.bias(l)), bits(hs.bias(l))), f"b {l}"
+        for r in (0, R - 1):
+            assert np.array_equal(bits(h.wgrad_of(l, r)), bits(hs.wgrad_of(l, r))), f"dW {l} {r}"
+    hs.close()
+    if lr >= 1e-6:
+        assert max(rel_err(W2[l] - Ws[l], 0 * Ws[l]) for l in range(L)) > 1e-4    # two updates have moved the weights
+        ref = oracle.mlp_step(nf, B, R, X, dY, W2, b2, lr)
+        acts = [h.activation(l) for l in range(L + 1)]
+        for l in range(L + 1):
+            assert close(acts[l], ref.acts[l], FP32_TOL), f"activation {l} of the third step"
+        ref = oracle.mlp_step(nf, B, R, X, dY, W2, b2, lr, given_acts=acts)   # backward on identical ReLU masks
+        assert close(h.dx(), ref.dX, FP32_TOL), "dX of the third step"
+        for l in range(L):
+            for r in (0, R - 1):
+                assert close(h.wgrad_of(l, r), ref.dW[r][l], FP32_TOL), f"dW layer {l} replica {r}"
+            assert close(h.weight(l), ref.W_new[l], FP32_TOL), f"W {l} after the third step"
+            assert close(h.bias(l), ref.b_new[l], FP32_TOL), f"b {l} after the third step"
+    h.close()
 
 
 def test_learning_rate_change_needs_no_new_graph_and_is_applied():
