@@ -358,7 +358,8 @@ bool small_model(const mi_mlp* h) {
   return true;
 }
 
-int op_update(mi_mlp* h, int l_or_all, float lr, hipStream_t s) {
+// beside_gemm: the launch shares the GPU with a GEMM of the same step on the other stream
+int op_update(mi_mlp* h, int l_or_all, float lr, hipStream_t s, bool beside_gemm = false) {
   TimedScope ts(h, s, MI_WGT_UPDATE, l_or_all >= 0 ? l_or_all : -1);
   if (ts.status) return ts.status;
   hipError_t e = hipSuccess;
@@ -385,7 +386,7 @@ int op_update(mi_mlp* h, int l_or_all, float lr, hipStream_t s) {
                                   h->stride, seg_end - bo, h->R)) {
       // the arena pads W_l to 64 floats, and rows * cols is a multiple of 64 here: b_l follows W_l directly
       e = mi::reduce_sgd_tiled(h->params + wo, h->params16 + wo, h->params16T + wo, h->grads + wo, rows, cols,
-                               h->stride, seg_end - bo, h->R, lr, s, h->neg_lr_dev);
+                               h->stride, seg_end - bo, h->R, lr, s, h->neg_lr_dev, beside_gemm);
     } else {
       e = mi::reduce_sgd(h->params + wo, h->params16 + wo, h->grads + wo, seg_end - wo, h->stride, h->R, lr, s,
                          h->neg_lr_dev);
@@ -613,7 +614,8 @@ int enqueue_step(mi_mlp* h, float lr) {
     if (per_layer) {
       hipStream_t su = dual ? s2 : h->stream2;
       if (!dual) MI_HIP(hipStreamWaitEvent(su, h->ev_layer[l], 0));
-      if ((rc = op_update(h, l, lr, su))) return rc;
+      // every layer's update but the last one's (layer 0) runs under the GEMMs of the layers below
+      if ((rc = op_update(h, l, lr, su, /*beside_gemm=*/su != s && l > 0))) return rc;
     }
   }
   if (dual || per_layer) {

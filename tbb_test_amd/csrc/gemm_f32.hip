@@ -1064,16 +1064,18 @@ __global__ __launch_bounds__(256) void gemm_f32_splitk_dma(GemmArgs p) {
 // The two backward GEMMs of one layer in one launch: the weight gradient (all replicas, bias
 // gradient fused) and the input gradient read the same dZ and depend on nothing of each other.  For
 // problems this small a step is a chain of launches of a few microseconds each, and one launch less
-// per layer is worth more than anything inside the kernels.  Workgroups [0, wgrad_blocks) run the
-// weight gradient (tile fastest, then replica), the rest the input gradient.
+// per layer is worth more than anything inside the kernels.  Workgroups [0, dgrad_blocks) run the
+// input gradient, the rest the weight gradient (tile fastest, then replica): a block of the input
+// gradient walks R times the K of a weight-gradient block, so the long blocks start first and the
+// short ones fill in behind them.
 template <int EPI_D>
-__global__ __launch_bounds__(256) void gemm_f32_splitk_pair(GemmArgs pw, GemmArgs pd, int wgrad_blocks) {
+__global__ __launch_bounds__(256) void gemm_f32_splitk_pair(GemmArgs pw, GemmArgs pd, int dgrad_blocks) {
   const int b = blockIdx.x;
-  if (b < wgrad_blocks) {
-    const int per = pw.tiles_m * pw.tiles_n, z = b / per;
-    splitk_block<false, false, EPI_NONE, true>(pw, b - z * per, z);
+  if (b < dgrad_blocks) {
+    splitk_block<true, false, EPI_D, false>(pd, b, 0);
   } else {
-    splitk_block<true, false, EPI_D, false>(pd, b - wgrad_blocks, 0);
+    const int per = pw.tiles_m * pw.tiles_n, w = b - dgrad_blocks, z = w / per;
+    splitk_block<false, false, EPI_NONE, true>(pw, w - z * per, z);
   }
 }
 
@@ -1386,8 +1388,8 @@ hipError_t sgemm_backward_pair(int R, int rows, int nout, int nin, const float* 
   pd.mask = mask; pd.ldmask = nin;
   pd.tiles_m = rows / 32; pd.tiles_n = nin / 32;
   const int wgrad_blocks = pw.tiles_m * pw.tiles_n * R, dgrad_blocks = pd.tiles_m * pd.tiles_n;
-  if (mask) launch_kernel(gemm_f32_splitk_pair<EPI_MASK>, dim3(wgrad_blocks + dgrad_blocks), dim3(256), 0, s, pw, pd, wgrad_blocks);
-  else launch_kernel(gemm_f32_splitk_pair<EPI_NONE>, dim3(wgrad_blocks + dgrad_blocks), dim3(256), 0, s, pw, pd, wgrad_blocks);
+  if (mask) launch_kernel(gemm_f32_splitk_pair<EPI_MASK>, dim3(wgrad_blocks + dgrad_blocks), dim3(256), 0, s, pw, pd, dgrad_blocks);
+  else launch_kernel(gemm_f32_splitk_pair<EPI_NONE>, dim3(wgrad_blocks + dgrad_blocks), dim3(256), 0, s, pw, pd, dgrad_blocks);
   return hipGetLastError();
 }
 

@@ -113,11 +113,13 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
 // floats that follow the matrix in W, W16 and every replica of G (a layer's bias and padding) are
 // updated the flat way by the same launch.  Needs rows and cols multiples of 64, tail a multiple
 // of 4 and 16-byte aligned pointers (reduce_sgd_tiled_fits); `stride` = floats between consecutive
-// replicas' gradients.
+// replicas' gradients.  beside_gemm: the launch will run next to a GEMM on another stream (one
+// workgroup per CU walks the tiles, see the launcher).
 bool reduce_sgd_tiled_fits(const float* W, const uint16_t* W16, const uint16_t* W16T, const float* G, int rows,
                            int cols, size_t stride, size_t tail, int R);
 hipError_t reduce_sgd_tiled(float* W, uint16_t* W16, uint16_t* W16T, const float* G, int rows, int cols, size_t stride,
-                            size_t tail, int R, float lr, hipStream_t s, const float* neg_lr_dev = nullptr);
+                            size_t tail, int R, float lr, hipStream_t s, const float* neg_lr_dev = nullptr,
+                            bool beside_gemm = false);
 
 // bf16: C = A[M,K] * B[N,K]^T with fp32 accumulation, both operands K-contiguous, blockIdx.z
 // batches with element strides batchA/B/C.  out_kind: 0 fp32 plain, 1 bf16 with bias + optional

@@ -169,19 +169,23 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
 // reference forwards the updated chunk to its consumers in the same pass that applies the SGD
 // update (mlp_omp.cc:240-252); here that pass writes, from registers, the fp32 master weights, the
 // bf16 copy, and -- through an LDS tile -- the transposed bf16 copy, so that no separate transpose
-// launch re-reads what the update just produced.  One workgroup per 64 x TC tile of W; a pass of
+// launch re-reads what the update just produced.  A workgroup takes the TR x TC tiles blockIdx.x,
+// blockIdx.x + gridDim.x, ... of W (one each when the grid covers them all); a pass of
 // the 256 threads covers 1024 / (TC/4) whole tile rows (TC = 256: four rows of 1 KB each, the
 // contiguous runs the memory likes), the arithmetic per element is that of reduce_sgd_vec4.  The
-// transposed copy leaves as runs of 128 bytes (64 rows of one column).  The workgroups of the
-// extra grid row blockIdx.y == rows / 64 update the `tail` floats that follow the matrix in the
-// arena (the layer's bias and padding) the flat way, so that a layer is one launch.
+// transposed copy leaves as runs of 128 bytes (64 rows of one column).  The tiles of one extra
+// tile row (tile_y == rows / TR) stand for the `tail` floats that follow the matrix in the
+// arena (the layer's bias and padding), updated the flat way, so that a layer is one launch.
+// GROUP = passes whose loads are in flight together.
 // Algorithmic traffic per weight: (R + 2) * 4 + 2 + 2 bytes.
-template <int R_FIXED, bool STREAM, int TR, int TC>
+template <int R_FIXED, bool STREAM, int TR, int TC, int GROUP>
 __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, unsigned short* __restrict__ W16,
                                                        unsigned short* __restrict__ W16T,
                                                        const float* __restrict__ G, int rows, int cols,
                                                        size_t stride, size_t tail, int R_dyn, float neg_lr_arg,
-                                                       const float* __restrict__ neg_lr_dev) {
+                                                       const float* __restrict__ neg_lr_dev, int tiles_x,
+                                                       int total_tiles) {
+  constexpr int NT = 256;  // threads of a workgroup
   // bf16 pairs; an odd number of words per row keeps the column gather below free of bank conflicts
   __shared__ unsigned int tile[TR][TC / 2 + 1];
   const int R = R_FIXED > 0 ? R_FIXED : R_dyn;
@@ -199,9 +203,11 @@ __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, un
     o[3] = fmaf(neg_lr, sum[3], w[3]);
     return o;
   };
-  if ((int)blockIdx.y * TR >= rows) {  // the floats behind the matrix: bias and padding
+  for (int t = blockIdx.x; t < total_tiles; t += gridDim.x) {
+  const int tile_x = t % tiles_x, tile_y = t / tiles_x;
+  if (tile_y * TR >= rows) {  // the floats behind the matrix: bias and padding
     const size_t base = (size_t)rows * cols, nvec = tail / 4;
-    for (size_t i = (size_t)blockIdx.x * 256 + tid; i < nvec; i += (size_t)gridDim.x * 256) {
+    for (size_t i = (size_t)tile_x * NT + tid; i < nvec; i += (size_t)tiles_x * NT) {
       const size_t off = base + i * 4;
       f32x4 sum = ld(G + off);
       for (int r = 1; r < R; ++r) sum += ld(G + (size_t)r * stride + off);
@@ -210,12 +216,11 @@ __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, un
       const u16x4 h = {f32_to_bf16_rne(o[0]), f32_to_bf16_rne(o[1]), f32_to_bf16_rne(o[2]), f32_to_bf16_rne(o[3])};
       *reinterpret_cast<u16x4*>(W16 + off) = h;
     }
-    return;
+    continue;
   }
-  const int r0 = blockIdx.y * TR, c0 = blockIdx.x * TC;
+  const int r0 = tile_y * TR, c0 = tile_x * TC;
   constexpr int VPR = TC / 4;            // float4 per tile row
-  constexpr int PASSES = TR * VPR / 256; // 256 float4 per pass
-  constexpr int GROUP = 4;               // passes whose loads are in flight together
+  constexpr int PASSES = TR * VPR / NT;  // NT float4 per pass; GROUP = passes whose loads are in flight together
   static_assert(PASSES % GROUP == 0, "tile shape");
 #pragma unroll 1
   for (int g = 0; g < PASSES / GROUP; ++g) {
@@ -223,7 +228,7 @@ __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, un
     f32x4 sum[GROUP], w[GROUP];
 #pragma unroll
     for (int i = 0; i < GROUP; ++i) {
-      const int idx = tid + 256 * (g * GROUP + i), row = idx / VPR, c4 = idx % VPR;
+      const int idx = tid + NT * (g * GROUP + i), row = idx / VPR, c4 = idx % VPR;
       off[i] = (size_t)(r0 + row) * cols + c0 + c4 * 4;
       sum[i] = ld(G + off[i]);
       w[i] = *reinterpret_cast<const f32x4*>(W + off[i]);
@@ -240,7 +245,7 @@ __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, un
     }
 #pragma unroll
     for (int i = 0; i < GROUP; ++i) {
-      const int idx = tid + 256 * (g * GROUP + i), row = idx / VPR, c4 = idx % VPR;
+      const int idx = tid + NT * (g * GROUP + i), row = idx / VPR, c4 = idx % VPR;
       const f32x4 o = update4(sum[i], w[i]);
       const u16x4 h = {f32_to_bf16_rne(o[0]), f32_to_bf16_rne(o[1]), f32_to_bf16_rne(o[2]), f32_to_bf16_rne(o[3])};
       *reinterpret_cast<f32x4*>(W + off[i]) = o;
@@ -254,13 +259,15 @@ __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, un
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
   constexpr int CP = TR / 8;  // 16-byte chunks per output row
 #pragma unroll
-  for (int i = 0; i < TC * CP / 256; ++i) {
-    const int q = tid + 256 * i, c = q / CP, part = q % CP;
+  for (int i = 0; i < TC * CP / NT; ++i) {
+    const int q = tid + NT * i, c = q / CP, part = q % CP;
     unsigned e[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) e[k] = (tile[part * 8 + k][c >> 1] >> ((c & 1) * 16)) & 0xffffu;
     const u32x4 v = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
     *reinterpret_cast<u32x4*>(W16T + (size_t)(c0 + c) * rows + r0 + part * 8) = v;
+  }
+  __syncthreads();  // the tile is read out before the next one is written
   }
 }
 
@@ -269,25 +276,44 @@ bool reduce_sgd_tiled_fits(const float* W, const uint16_t* W16, const uint16_t* 
   auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   return rows > 0 && cols > 0 && rows % 64 == 0 && cols % 64 == 0 && al16(W) && al16(G) && al16(W16T) &&
          (reinterpret_cast<uintptr_t>(W16) & 7) == 0 && (stride % 4 == 0 || R == 1) && tail % 4 == 0 &&
-         rows / 64 < 65535;
+         (long long)(rows / 64 + 1) * (cols / 64) < (1ll << 31);
 }
 
 hipError_t reduce_sgd_tiled(float* W, uint16_t* W16, uint16_t* W16T, const float* G, int rows, int cols, size_t stride,
-                            size_t tail, int R, float lr, hipStream_t s, const float* neg_lr_dev) {
+                            size_t tail, int R, float lr, hipStream_t s, const float* neg_lr_dev, bool beside_gemm) {
   if (!reduce_sgd_tiled_fits(W, W16, W16T, G, rows, cols, stride, tail, R) || R <= 0) return hipErrorInvalidValue;
   const float neg_lr = -lr;
   const bool stream = (double)(R + 1) * (double)rows * (double)cols * 4.0 > 192e6;  // beyond the Infinity Cache
   // 64 x 64 tiles; 64 x 256, 128 x 128 and 256 x 64 tiles and non-temporal stores were measured on
   // 8192 x 8192 layers with R = 4 and change nothing (2.83-2.93 ms for 8 layers, 5.0-5.1 TB/s): the
   // mix of five read and three write streams is what the memory sustains.
-  const dim3 grid(cols / 64, rows / 64 + (tail ? 1 : 0));
-#define MI_LAUNCH_TILE3(RF, ST, TR, TC)                                                                          \
-  launch_kernel((reduce_sgd_tile<RF, ST, TR, TC>), grid, dim3(256), 0, s, W, W16, W16T, G, rows, cols, stride, tail, \
-                R, neg_lr, neg_lr_dev)
+  const int tiles_x = cols / 64, total_tiles = tiles_x * (rows / 64 + (tail ? 1 : 0));
+  // A launch that runs beside a GEMM on another stream (the per-layer update of a bf16 model under
+  // the input-gradient GEMM of the next layer) is one workgroup per CU walking the tiles, with half
+  // the loads in flight (65 instead of 120 registers at R = 4): that leaves the registers and the
+  // LDS a 256 x 256 GEMM workgroup needs on the same CU, where thousands of short workgroups take
+  // whole CUs in turns with the GEMM.  Alone such a grid is as fast as the full one (2.90 against
+  // 2.86 ms for eight 8192 x 8192 layers, R = 4); beside the GEMMs the step of that model takes
+  // 40.2-40.3 ms instead of 40.8-40.9.  Twice or half as many workgroups, or workgroups of 64 or
+  // 128 threads that stay longer, lose the gain or more: a GEMM runs slower for as long as an
+  // update runs on its CUs, so the update has to be short.
+  int grid_x = total_tiles;
+  if (beside_gemm && stream) {
+    int dev = 0, cus = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+    if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev); e != hipSuccess) return e;
+    if (cus > 0 && cus < grid_x) grid_x = cus;
+  }
+  const bool lean = grid_x < total_tiles;
+  const dim3 grid(grid_x);
+#define MI_LAUNCH_TILE3(RF, ST, TR, TC, GR)                                                                          \
+  launch_kernel((reduce_sgd_tile<RF, ST, TR, TC, GR>), grid, dim3(256), 0, s, W, W16, W16T, G, rows, cols, stride, tail, \
+                R, neg_lr, neg_lr_dev, tiles_x, total_tiles)
 #define MI_LAUNCH_TILE(RF)                     \
   do {                                         \
-    if (stream) MI_LAUNCH_TILE3(RF, true, 64, 64);      \
-    else MI_LAUNCH_TILE3(RF, false, 64, 64);                 \
+    if (lean) MI_LAUNCH_TILE3(RF, true, 64, 64, 2);      \
+    else if (stream) MI_LAUNCH_TILE3(RF, true, 64, 64, 4);      \
+    else MI_LAUNCH_TILE3(RF, false, 64, 64, 4);                 \
   } while (0)
   switch (R) {
     case 1: MI_LAUNCH_TILE(1); break;
