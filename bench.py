@@ -146,6 +146,7 @@ def main():
     ap.add_argument("--hvariant", type=int, default=0, help="tuning: forced bf16 GEMM tile variant")
     ap.add_argument("--variants", default="", help="tuning: forced GEMM tile variants 'nt,nn,tn'")
     ap.add_argument("--serial-backward", action="store_true", help="whole backward pass on one stream")
+    ap.add_argument("--no-graph", action="store_true", help="tuning: every step launched eagerly instead of replaying its graph")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--gemm", default="", metavar="M,N,K",
                     help="instead of the training step: time the forward-type GEMM entry point alone (mi_hgemm_nt / "
@@ -172,6 +173,8 @@ def main():
 
     X, Ws, dY = hostlib.init_problem(nf, B, R, args.seed)
     flags = (0 if args.flat_update else capi.FLAG_PER_LAYER_UPDATE) | (capi.FLAG_SERIAL_BACKWARD if args.serial_backward else 0)
+    if args.no_graph:
+        flags |= capi.FLAG_NO_GRAPH
     h = capi.MlpHandle(nf, B, R, dtype=capi.MI_BF16 if dtype == "bf16" else capi.MI_F32, flags=flags)
     if args.hvariant:
         capi.check(capi.lib().mi_set_hgemm_variant(args.hvariant))
