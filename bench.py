@@ -10,7 +10,9 @@ the timed region starts.  Default schedule: the weight-gradient GEMMs and the pe
 launches trail the chain of input-gradient GEMMs on a second stream.  The timed loop is the
 reference's: K consecutive steps, each on the weights the step before left, with the reference's
 learning rate of 1e-10 (mlp_omp.cc:435-737 with alpha at :609,699,718,729), at which the
-sum-reduced updates stay finite however many steps are run.
+sum-reduced updates stay finite however many steps are run (--lr 0.01 --restore-each-step times
+the same step at the learning rate of the parity tests, with a device copy of the weights added
+to every step).
 
 Prints one JSON line:
   value          whole-step throughput, TFLOP/s on the reference's FLOP model
@@ -140,6 +142,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
     ap.add_argument("--lr", type=float, default=1e-10, help="learning rate (default: the reference benchmark's alpha)")
+    ap.add_argument("--restore-each-step", action="store_true",
+                    help="start every step from the initial weights (a device copy inside the timed region): "
+                         "keeps a loop at a visible learning rate such as 0.01 finite")
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--flat-update", action="store_true",
                     help="one update launch at the end of the step instead of per-layer updates on the second stream")
@@ -189,6 +194,8 @@ def main():
     params, _ = h.param_count()
 
     def one_step():
+        if args.restore_each_step:
+            h.restore_weights()
         h.step(args.lr)
 
     # Untimed spin-up so that the GPU has left its idle clock state before anything is measured
@@ -281,7 +288,9 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.config}: {layers} FC layers, widths "
                                + (f"{nf[0]} throughout" if len(set(nf)) == 1 else " ".join(str(v) for v in nf))
-                               + f", ReLU between layers, batch {B} per replica x {R} replicas, lr {args.lr}, seed {args.seed}",
+                               + f", ReLU between layers, batch {B} per replica x {R} replicas, "
+                               + ("every step from the initial weights" if args.restore_each_step else "consecutive steps")
+                               + f", lr {args.lr}, seed {args.seed}",
                    "schedule": schedule, "device": info["name"], "num_cus": info["num_cus"]},
         "gemm_flop_per_step": gemm_flop_step,
         "phase_ms_per_step": {k: round(v, 4) for k, v in per_phase.items()},
