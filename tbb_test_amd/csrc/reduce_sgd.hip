@@ -204,70 +204,70 @@ __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, un
     return o;
   };
   for (int t = blockIdx.x; t < total_tiles; t += gridDim.x) {
-  const int tile_x = t % tiles_x, tile_y = t / tiles_x;
-  if (tile_y * TR >= rows) {  // the floats behind the matrix: bias and padding
-    const size_t base = (size_t)rows * cols, nvec = tail / 4;
-    for (size_t i = (size_t)tile_x * NT + tid; i < nvec; i += (size_t)tiles_x * NT) {
-      const size_t off = base + i * 4;
-      f32x4 sum = ld(G + off);
-      for (int r = 1; r < R; ++r) sum += ld(G + (size_t)r * stride + off);
-      const f32x4 o = update4(sum, *reinterpret_cast<const f32x4*>(W + off));
-      *reinterpret_cast<f32x4*>(W + off) = o;
-      const u16x4 h = {f32_to_bf16_rne(o[0]), f32_to_bf16_rne(o[1]), f32_to_bf16_rne(o[2]), f32_to_bf16_rne(o[3])};
-      *reinterpret_cast<u16x4*>(W16 + off) = h;
+    const int tile_x = t % tiles_x, tile_y = t / tiles_x;
+    if (tile_y * TR >= rows) {  // the floats behind the matrix: bias and padding
+      const size_t base = (size_t)rows * cols, nvec = tail / 4;
+      for (size_t i = (size_t)tile_x * NT + tid; i < nvec; i += (size_t)tiles_x * NT) {
+        const size_t off = base + i * 4;
+        f32x4 sum = ld(G + off);
+        for (int r = 1; r < R; ++r) sum += ld(G + (size_t)r * stride + off);
+        const f32x4 o = update4(sum, *reinterpret_cast<const f32x4*>(W + off));
+        *reinterpret_cast<f32x4*>(W + off) = o;
+        const u16x4 h = {f32_to_bf16_rne(o[0]), f32_to_bf16_rne(o[1]), f32_to_bf16_rne(o[2]), f32_to_bf16_rne(o[3])};
+        *reinterpret_cast<u16x4*>(W16 + off) = h;
+      }
+      continue;
     }
-    continue;
-  }
-  const int r0 = tile_y * TR, c0 = tile_x * TC;
-  constexpr int VPR = TC / 4;            // float4 per tile row
-  constexpr int PASSES = TR * VPR / NT;  // NT float4 per pass; GROUP = passes whose loads are in flight together
-  static_assert(PASSES % GROUP == 0, "tile shape");
+    const int r0 = tile_y * TR, c0 = tile_x * TC;
+    constexpr int VPR = TC / 4;            // float4 per tile row
+    constexpr int PASSES = TR * VPR / NT;  // NT float4 per pass; GROUP = passes whose loads are in flight together
+    static_assert(PASSES % GROUP == 0, "tile shape");
 #pragma unroll 1
-  for (int g = 0; g < PASSES / GROUP; ++g) {
-    size_t off[GROUP];
-    f32x4 sum[GROUP], w[GROUP];
+    for (int g = 0; g < PASSES / GROUP; ++g) {
+      size_t off[GROUP];
+      f32x4 sum[GROUP], w[GROUP];
 #pragma unroll
-    for (int i = 0; i < GROUP; ++i) {
-      const int idx = tid + NT * (g * GROUP + i), row = idx / VPR, c4 = idx % VPR;
-      off[i] = (size_t)(r0 + row) * cols + c0 + c4 * 4;
-      sum[i] = ld(G + off[i]);
-      w[i] = *reinterpret_cast<const f32x4*>(W + off[i]);
+      for (int i = 0; i < GROUP; ++i) {
+        const int idx = tid + NT * (g * GROUP + i), row = idx / VPR, c4 = idx % VPR;
+        off[i] = (size_t)(r0 + row) * cols + c0 + c4 * 4;
+        sum[i] = ld(G + off[i]);
+        w[i] = *reinterpret_cast<const f32x4*>(W + off[i]);
+      }
+      if (R_FIXED > 0) {
+#pragma unroll
+        for (int r = 1; r < R_FIXED; ++r)
+#pragma unroll
+          for (int i = 0; i < GROUP; ++i) sum[i] += ld(G + (size_t)r * stride + off[i]);
+      } else {
+        for (int r = 1; r < R; ++r)
+#pragma unroll
+          for (int i = 0; i < GROUP; ++i) sum[i] += ld(G + (size_t)r * stride + off[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < GROUP; ++i) {
+        const int idx = tid + NT * (g * GROUP + i), row = idx / VPR, c4 = idx % VPR;
+        const f32x4 o = update4(sum[i], w[i]);
+        const u16x4 h = {f32_to_bf16_rne(o[0]), f32_to_bf16_rne(o[1]), f32_to_bf16_rne(o[2]), f32_to_bf16_rne(o[3])};
+        *reinterpret_cast<f32x4*>(W + off[i]) = o;
+        *reinterpret_cast<u16x4*>(W16 + off[i]) = h;
+        tile[row][c4 * 2] = (unsigned)h[0] | ((unsigned)h[1] << 16);
+        tile[row][c4 * 2 + 1] = (unsigned)h[2] | ((unsigned)h[3] << 16);
+      }
     }
-    if (R_FIXED > 0) {
+    __syncthreads();
+    // transposed copy: output row c0 + c holds the tile's TR rows = 2 TR contiguous bytes, 16 per thread
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    constexpr int CP = TR / 8;  // 16-byte chunks per output row
 #pragma unroll
-      for (int r = 1; r < R_FIXED; ++r)
+    for (int i = 0; i < TC * CP / NT; ++i) {
+      const int q = tid + NT * i, c = q / CP, part = q % CP;
+      unsigned e[8];
 #pragma unroll
-        for (int i = 0; i < GROUP; ++i) sum[i] += ld(G + (size_t)r * stride + off[i]);
-    } else {
-      for (int r = 1; r < R; ++r)
-#pragma unroll
-        for (int i = 0; i < GROUP; ++i) sum[i] += ld(G + (size_t)r * stride + off[i]);
+      for (int k = 0; k < 8; ++k) e[k] = (tile[part * 8 + k][c >> 1] >> ((c & 1) * 16)) & 0xffffu;
+      const u32x4 v = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+      *reinterpret_cast<u32x4*>(W16T + (size_t)(c0 + c) * rows + r0 + part * 8) = v;
     }
-#pragma unroll
-    for (int i = 0; i < GROUP; ++i) {
-      const int idx = tid + NT * (g * GROUP + i), row = idx / VPR, c4 = idx % VPR;
-      const f32x4 o = update4(sum[i], w[i]);
-      const u16x4 h = {f32_to_bf16_rne(o[0]), f32_to_bf16_rne(o[1]), f32_to_bf16_rne(o[2]), f32_to_bf16_rne(o[3])};
-      *reinterpret_cast<f32x4*>(W + off[i]) = o;
-      *reinterpret_cast<u16x4*>(W16 + off[i]) = h;
-      tile[row][c4 * 2] = (unsigned)h[0] | ((unsigned)h[1] << 16);
-      tile[row][c4 * 2 + 1] = (unsigned)h[2] | ((unsigned)h[3] << 16);
-    }
-  }
-  __syncthreads();
-  // transposed copy: output row c0 + c holds the tile's TR rows = 2 TR contiguous bytes, 16 per thread
-  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-  constexpr int CP = TR / 8;  // 16-byte chunks per output row
-#pragma unroll
-  for (int i = 0; i < TC * CP / NT; ++i) {
-    const int q = tid + NT * i, c = q / CP, part = q % CP;
-    unsigned e[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) e[k] = (tile[part * 8 + k][c >> 1] >> ((c & 1) * 16)) & 0xffffu;
-    const u32x4 v = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
-    *reinterpret_cast<u32x4*>(W16T + (size_t)(c0 + c) * rows + r0 + part * 8) = v;
-  }
-  __syncthreads();  // the tile is read out before the next one is written
+    __syncthreads();  // the tile is read out before the next one is written
   }
 }
 
