@@ -27,7 +27,9 @@ __device__ __forceinline__ unsigned short f32_to_bf16_rne(float f) {
 
 // UNROLL float4 per thread per trip.  Two regimes, chosen by the launcher from the bytes moved:
 //   STREAM = true   the arenas exceed the 256 MB Infinity Cache: the gradients are read exactly
-//                   once, so they are loaded non-temporally; one float4 per thread, one trip.
+//                   once, so they are loaded non-temporally; four float4 per thread in flight, one
+//                   trip (R = 8, 3.36 GB: 5.70 TB/s with one, 5.98 with two, 6.09 with four, 3.98
+//                   with eight; R = 2, 1.07 GB: 6.64 / 6.67 / 6.73 / 5.76).
 //   STREAM = false  everything fits the Infinity Cache, where the gradient GEMMs have just left
 //                   their output: ordinary loads (non-temporal ones would bypass that cache), two
 //                   float4 per thread in flight.
@@ -122,12 +124,12 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
     // cached regime: about a thousand blocks for a launch over a whole arena (2048 float4 each;
     // measured 32.4 us against 33.3 us with 512 at config 2), 512 float4 per block below that, so
     // that a single layer's launch still covers the CUs
-    const size_t per_block = stream ? 256 : (nvec >= ((size_t)1 << 21) ? 2048 : 512);
+    const size_t per_block = stream ? 1024 : (nvec >= ((size_t)1 << 21) ? 2048 : 512);
     const int blocks = grid_for(nvec, (int)per_block, stream ? (1 << 30) : 8192);
 #define MI_LAUNCH_REDUCE2(RF, BF)                                                                          \
   do {                                                                                                     \
     if (stream)                                                                                            \
-      launch_kernel((reduce_sgd_vec4<RF, BF, 1, true>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, \
+      launch_kernel((reduce_sgd_vec4<RF, BF, 4, true>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, \
                          stride / 4, R, neg_lr, neg_lr_dev);                                               \
     else                                                                                                   \
       launch_kernel((reduce_sgd_vec4<RF, BF, 2, false>), dim3(blocks), dim3(256), 0, s, W, W16, G, nvec, \
