@@ -885,11 +885,18 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
 // the registers the MFMAs read -- no LDS tile, no barrier in the loop (the operands of such small
 // problems sit in the L2).  The four partial blocks are added through the LDS in wavefront order
 // (deterministic), wavefront w finishing rows 8w .. 8w+7 of the block.
-// `tile` = index of the 32 x 32 block in row-major order, `z` = batch entry.
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM>
-__device__ __forceinline__ void splitk_block(const GemmArgs& p, int tile, int z) {
-  __shared__ float part[4][16][64];
-  __shared__ float cs_part[4][32];
+// NW = 8 (the forward GEMM from K = 512 on, see splitk_eight_waves): eight wavefronts, two per SIMD,
+// with an eighth of K each -- half the chain of dependent MFMAs per wavefront, which is what a
+// launch of one workgroup per CU waits for; wavefront w then finishes the accumulator registers
+// 2w and 2w+1.
+// `tile` = index of the 32 x 32 block in row-major order, `z` = batch entry, `lds` = the
+// workgroup's SPLITK_LDS_FLOATS(NW) floats of LDS.
+#define SPLITK_LDS_FLOATS(NW) ((NW) * 16 * 64 + (NW) * 32)
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM, int NW = 4>
+__device__ __forceinline__ void splitk_block(const GemmArgs& p, int tile, int z, float* lds) {
+  static_assert(NW == 4 || NW == 8, "split of K over the wavefronts");
+  float(*part)[16][64] = reinterpret_cast<float(*)[16][64]>(lds);             // [NW][16][64]
+  float(*cs_part)[32] = reinterpret_cast<float(*)[32]>(lds + NW * 16 * 64);  // [NW][32]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hi = lane >> 5;
   const int tile_m = tile / p.tiles_n, tile_n = tile - tile_m * p.tiles_n;
@@ -897,7 +904,7 @@ __device__ __forceinline__ void splitk_block(const GemmArgs& p, int tile, int z)
   const float* __restrict__ A = p.A + (size_t)z * p.batchA;
   const float* __restrict__ B = p.B + (size_t)z * p.batchB;
   float* __restrict__ C = p.C + (size_t)z * p.batchC;
-  const int kq = p.K / 4, k_begin = wave * kq, chunks = kq / 8;
+  const int kq = p.K / NW, k_begin = wave * kq, chunks = kq / 8;
   // lane (l32, hi) feeds MFMA step q of a chunk with k = chunk*8 + 4*hi + q
   const float* a_ptr = A_KMAJOR ? A + (size_t)(m0 + l32) * p.lda + k_begin + 4 * hi
                                 : A + (size_t)(k_begin + 4 * hi) * p.lda + m0 + l32;
@@ -951,16 +958,21 @@ __device__ __forceinline__ void splitk_block(const GemmArgs& p, int tile, int z)
     if (hi == 0) cs_part[wave][l32] = cs;
   }
   __syncthreads();
-  if (COLSUM && do_colsum && tid < 32)
-    p.colsum[(size_t)z * p.batchColsum + m0 + tid] =
-        ((cs_part[0][tid] + cs_part[1][tid]) + cs_part[2][tid]) + cs_part[3][tid];
+  if (COLSUM && do_colsum && tid < 32) {
+    float total = cs_part[0][tid];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) total += cs_part[w][tid];
+    p.colsum[(size_t)z * p.batchColsum + m0 + tid] = total;
+  }
   const int col = n0 + l32;
   const float bias_v = (EPI == EPI_BIAS_RELU && p.bias) ? p.bias[col] : 0.0f;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const int r = 4 * wave + e;
-    float v = ((part[0][r][lane] + part[1][r][lane]) + part[2][r][lane]) + part[3][r][lane];
-    const int row = m0 + 8 * wave + 4 * hi + e;  // register r holds row 8*(r/4) + 4*hi + r%4
+  for (int e = 0; e < 16 / NW; ++e) {
+    const int r = (16 / NW) * wave + e;
+    float v = part[0][r][lane];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) v += part[w][r][lane];
+    const int row = m0 + 8 * (r / 4) + 4 * hi + (r % 4);  // register r holds row 8*(r/4) + 4*hi + r%4
     if (EPI == EPI_BIAS_RELU) {
       v += bias_v;
       if (p.relu) v = v > 0.0f ? v : 0.0f;
@@ -971,9 +983,17 @@ __device__ __forceinline__ void splitk_block(const GemmArgs& p, int tile, int z)
   }
 }
 
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM>
-__global__ __launch_bounds__(256) void gemm_f32_splitk(GemmArgs p) {
-  splitk_block<A_KMAJOR, B_KMAJOR, EPI, COLSUM>(p, blockIdx.x, blockIdx.z);
+// Eight wavefronts for the forward GEMM (both operands K-contiguous) when every wavefront still
+// gets whole sub-blocks of the direct-load kernel below: the two kernels add the same partial sums
+// in the same order and give the same bits.
+static inline bool splitk_eight_waves(bool a_kmajor, bool b_kmajor, int K) {
+  return a_kmajor && b_kmajor && K >= 512 && K % 256 == 0;
+}
+
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_f32_splitk(GemmArgs p) {
+  __shared__ float lds[SPLITK_LDS_FLOATS(NW)];
+  splitk_block<A_KMAJOR, B_KMAJOR, EPI, COLSUM, NW>(p, blockIdx.x, blockIdx.z, lds);
 }
 
 // The split-K kernel for two K-contiguous operands (the forward GEMM) with direct-to-LDS loads.
@@ -983,34 +1003,40 @@ __global__ __launch_bounds__(256) void gemm_f32_splitk(GemmArgs p) {
 // there is no barrier in the loop: sub-blocks of 64 k (8 KB per operand) travel through two
 // buffers, the wavefront waits for its own loads (vmcnt) and multiplies from the LDS (rows of 256
 // bytes, 16-byte chunks XOR-swizzled with the row so that fragment reads touch every bank once).
-template <int EPI>
-__global__ __launch_bounds__(256) void gemm_f32_splitk_dma(GemmArgs p) {
+// NW = 8, SW = 32: eight wavefronts with an eighth of K each and sub-blocks of 32 k (rows of 128
+// bytes, 8 rows per load instruction), the same 128 KB of LDS: half the chain of dependent MFMAs
+// per wavefront (K = 512: 32 instead of 64), which is what a launch of one workgroup per CU waits for.
+template <int EPI, int NW, int SW>
+__global__ __launch_bounds__(NW * 64) void gemm_f32_splitk_dma(GemmArgs p) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  constexpr int SW = 64;              // k per sub-block
-  constexpr int SB = 32 * SW;         // floats of one operand's sub-block
+  constexpr int SB = 32 * SW;         // floats of one operand's sub-block (SW = k per sub-block)
+  constexpr int CH = SW / 4;          // 16-byte chunks per row
+  constexpr int RPI = 64 / CH;        // rows one load instruction covers
+  constexpr int NI = 32 / RPI;        // load instructions per operand and sub-block
+  static_assert(NW * 4 * SB * sizeof(float) <= 128 * 1024 && (CH == 8 || CH == 16), "sub-block shape");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hi = lane >> 5;
   const int tile_m = blockIdx.x / p.tiles_n, tile_n = blockIdx.x - tile_m * p.tiles_n;
   const int m0 = tile_m * 32, n0 = tile_n * 32;
-  const int kq = p.K / 4, nsb = kq / SW;
+  const int kq = p.K / NW, nsb = kq / SW;
   float* region = smem + wave * (4 * SB);  // [buffer][A | B]
   const unsigned lds_base = (unsigned)(size_t)((__attribute__((address_space(3))) const void*)region);
-  // load instruction j covers rows 4j .. 4j+3; lane i fills chunk position i % 16 of row 4j + i / 16
-  unsigned offa[8], offb[8];
+  // load instruction j covers rows RPI j .. RPI j + RPI - 1; lane i fills chunk position i % CH of row RPI j + i / CH
+  unsigned offa[NI], offb[NI];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int row = 4 * j + (lane >> 4), pos = lane & 15;
-    offa[j] = 4u * ((unsigned)row * (unsigned)p.lda + (unsigned)((pos ^ (row & 15)) * 4));
-    offb[j] = 4u * ((unsigned)row * (unsigned)p.ldb + (unsigned)((pos ^ (row & 15)) * 4));
+  for (int j = 0; j < NI; ++j) {
+    const int row = RPI * j + lane / CH, pos = lane % CH;
+    offa[j] = 4u * ((unsigned)row * (unsigned)p.lda + (unsigned)((pos ^ (row & (CH - 1))) * 4));
+    offb[j] = 4u * ((unsigned)row * (unsigned)p.ldb + (unsigned)((pos ^ (row & (CH - 1))) * 4));
   }
   const float* a_base = p.A + (size_t)m0 * p.lda + (size_t)wave * kq;
   const float* b_base = p.B + (size_t)n0 * p.ldb + (size_t)wave * kq;
   auto issue = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) load_to_lds_f32(a_base, offa[j], lds_base + 4u * (unsigned)(buf * 2 * SB + j * 256));
+    for (int j = 0; j < NI; ++j) load_to_lds_f32(a_base, offa[j], lds_base + 4u * (unsigned)(buf * 2 * SB + j * 256));
 #pragma unroll
-    for (int j = 0; j < 8; ++j) load_to_lds_f32(b_base, offb[j], lds_base + 4u * (unsigned)(buf * 2 * SB + SB + j * 256));
+    for (int j = 0; j < NI; ++j) load_to_lds_f32(b_base, offb[j], lds_base + 4u * (unsigned)(buf * 2 * SB + SB + j * 256));
     a_base += SW;
     b_base += SW;
   };
@@ -1021,14 +1047,14 @@ __global__ __launch_bounds__(256) void gemm_f32_splitk_dma(GemmArgs p) {
   if (nsb > 1) issue(1);
   for (int sb = 0; sb < nsb; ++sb) {
     const int cur = sb & 1;
-    if (sb + 1 < nsb) __builtin_amdgcn_s_waitcnt(vmcnt_only(16));  // the younger sub-block may stay in flight
+    if (sb + 1 < nsb) __builtin_amdgcn_s_waitcnt(vmcnt_only(2 * NI));  // the younger sub-block may stay in flight
     else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
     asm volatile("" ::: "memory");
     const float* a_tile = region + cur * 2 * SB + l32 * SW;
     const float* b_tile = a_tile + SB;
 #pragma unroll
     for (int kk = 0; kk < SW / 8; ++kk) {
-      const int chunk = ((2 * kk + hi) ^ (l32 & 15)) * 4;
+      const int chunk = ((2 * kk + hi) ^ (l32 & (CH - 1))) * 4;
       const f32x4 fa = *reinterpret_cast<const f32x4*>(a_tile + chunk);
       const f32x4 fb = *reinterpret_cast<const f32x4*>(b_tile + chunk);
 #pragma unroll
@@ -1040,7 +1066,7 @@ __global__ __launch_bounds__(256) void gemm_f32_splitk_dma(GemmArgs p) {
       issue(cur);
     }
   }
-  // add the four partial blocks in wavefront order, as the register-loading kernel does
+  // add the partial blocks in wavefront order, as the register-loading kernel does
   __syncthreads();
   float(*part)[16][64] = reinterpret_cast<float(*)[16][64]>(smem);
 #pragma unroll
@@ -1049,10 +1075,12 @@ __global__ __launch_bounds__(256) void gemm_f32_splitk_dma(GemmArgs p) {
   const int col = n0 + l32;
   const float bias_v = (EPI == EPI_BIAS_RELU && p.bias) ? p.bias[col] : 0.0f;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const int r = 4 * wave + e;
-    float v = ((part[0][r][lane] + part[1][r][lane]) + part[2][r][lane]) + part[3][r][lane];
-    const int row = m0 + 8 * wave + 4 * hi + e;
+  for (int e = 0; e < 16 / NW; ++e) {
+    const int r = (16 / NW) * wave + e;
+    float v = part[0][r][lane];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) v += part[w][r][lane];
+    const int row = m0 + 8 * (r / 4) + 4 * hi + (r % 4);  // register r holds row 8*(r/4) + 4*hi + r%4
     if (EPI == EPI_BIAS_RELU) {
       v += bias_v;
       if (p.relu) v = v > 0.0f ? v : 0.0f;
@@ -1070,12 +1098,13 @@ __global__ __launch_bounds__(256) void gemm_f32_splitk_dma(GemmArgs p) {
 // short ones fill in behind them.
 template <int EPI_D>
 __global__ __launch_bounds__(256) void gemm_f32_splitk_pair(GemmArgs pw, GemmArgs pd, int dgrad_blocks) {
+  __shared__ float lds[SPLITK_LDS_FLOATS(4)];  // one region for either kind of block
   const int b = blockIdx.x;
   if (b < dgrad_blocks) {
-    splitk_block<true, false, EPI_D, false>(pd, b, 0);
+    splitk_block<true, false, EPI_D, false>(pd, b, 0, lds);
   } else {
     const int per = pw.tiles_m * pw.tiles_n, w = b - dgrad_blocks, z = w / per;
-    splitk_block<false, false, EPI_NONE, true>(pw, w - z * per, z);
+    splitk_block<false, false, EPI_NONE, true>(pw, w - z * per, z, lds);
   }
 }
 
@@ -1191,19 +1220,29 @@ template <bool AK, bool BKM, int EPI, bool COLSUM>
 static hipError_t launch_splitk(GemmArgs& p, int batch, hipStream_t s) {
   p.tiles_m = p.M / 32;
   p.tiles_n = p.N / 32;
-  launch_kernel((gemm_f32_splitk<AK, BKM, EPI, COLSUM>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0, s, p);
+  if (splitk_eight_waves(AK, BKM, p.K))
+    launch_kernel((gemm_f32_splitk<AK, BKM, EPI, COLSUM, 8>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(512), 0, s, p);
+  else
+    launch_kernel((gemm_f32_splitk<AK, BKM, EPI, COLSUM, 4>), dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(256), 0, s, p);
   return hipGetLastError();
 }
 
 template <int EPI>
 static hipError_t launch_splitk_dma(GemmArgs& p, hipStream_t s) {
-  constexpr size_t lds_bytes = 4 * 4 * 32 * 64 * sizeof(float);  // 4 wavefronts x 2 buffers x 2 operands x 8 KB
-  auto kern = gemm_f32_splitk_dma<EPI>;
-  static LdsOptIn opt_in;
-  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) return e;
+  constexpr size_t lds_bytes = 4 * 4 * 32 * 64 * sizeof(float);  // wavefronts x 2 buffers x 2 operands x sub-block: 128 KB either way
   p.tiles_m = p.M / 32;
   p.tiles_n = p.N / 32;
-  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n), dim3(256), lds_bytes, s, p);
+  if (splitk_eight_waves(true, true, p.K)) {
+    auto kern = gemm_f32_splitk_dma<EPI, 8, 32>;
+    static LdsOptIn opt_in;
+    if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) return e;
+    launch_kernel(kern, dim3(p.tiles_m * p.tiles_n), dim3(512), lds_bytes, s, p);
+  } else {
+    auto kern = gemm_f32_splitk_dma<EPI, 4, 64>;
+    static LdsOptIn opt_in;
+    if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) return e;
+    launch_kernel(kern, dim3(p.tiles_m * p.tiles_n), dim3(256), lds_bytes, s, p);
+  }
   return hipGetLastError();
 }
 
