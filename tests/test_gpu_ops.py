@@ -82,8 +82,10 @@ def run_tn(dZ, A, R, variant=0, with_colsum=True):
 GEMM_SHAPES = [
     (128, 128, 32), (256, 128, 64), (128, 256, 96), (512, 512, 512), (384, 640, 160),
     (64, 64, 32), (192, 64, 64),
-    # split-K kernel with direct-to-LDS loads (forward GEMM, K a multiple of 256): one, two and five sub-blocks per wavefront
-    (64, 96, 256), (512, 512, 512), (96, 64, 1280),
+    # split-K kernel with direct-to-LDS loads (forward GEMM, K a multiple of 256): four wavefronts and
+    # one sub-block of 64 k each at K = 256; from K = 512 on eight wavefronts with two, three, five and
+    # eight sub-blocks of 32 k each
+    (64, 96, 256), (512, 512, 512), (64, 64, 768), (96, 64, 1280), (32, 32, 2048),
     # tile grids whose XCD-aware orders divide by something that is not a power of two:
     # 8 x 3 tiles (contiguous range per XCD), 32 x 24 tiles (super-tiles, 3 per row)
     (1024, 384, 64), (4096, 3072, 32),
