@@ -892,7 +892,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f32_dma(GemmArgs p) {
 // `tile` = index of the 32 x 32 block in row-major order, `z` = batch entry, `lds` = the
 // workgroup's SPLITK_LDS_FLOATS(NW) floats of LDS.
 #define SPLITK_LDS_FLOATS(NW) ((NW) * 16 * 64 + (NW) * 32)
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM, int NW = 4>
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool COLSUM, int NW = 4, int DEPTH = 4>
 __device__ __forceinline__ void splitk_block(const GemmArgs& p, int tile, int z, float* lds) {
   static_assert(NW == 4 || NW == 8, "split of K over the wavefronts");
   float(*part)[16][64] = reinterpret_cast<float(*)[16][64]>(lds);             // [NW][16][64]
@@ -925,7 +925,6 @@ __device__ __forceinline__ void splitk_block(const GemmArgs& p, int tile, int z,
   for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
   const bool do_colsum = COLSUM && p.colsum != nullptr && tile_n == 0;
   float cs = 0.0f;
-  constexpr int DEPTH = 4;  // chunks in flight (8 measured: no gain)
   float fa[DEPTH][4], fb[DEPTH][4];
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d)
@@ -1096,15 +1095,22 @@ __global__ __launch_bounds__(NW * 64) void gemm_f32_splitk_dma(GemmArgs p) {
 // input gradient, the rest the weight gradient (tile fastest, then replica): a block of the input
 // gradient walks R times the K of a weight-gradient block, so the long blocks start first and the
 // short ones fill in behind them.
+// Chunks of 8 k a wavefront of the paired launch requests ahead.  With three workgroups per CU
+// the other eleven wavefronts of the CU cover a wavefront's wait, and every request more in flight
+// (3 072 wavefronts ask at once) makes the launch slower: config 1 step 59.4 us with four chunks
+// ahead, 58.5 with three, 57.3 with two, 53.7 with one, 62.9-66.5 with eight.  The separate
+// launches (one or two workgroups per CU) keep four: with two their input gradient takes 24.5
+// instead of 21 us.
+constexpr int PAIR_DEPTH = 1;
 template <int EPI_D>
 __global__ __launch_bounds__(256) void gemm_f32_splitk_pair(GemmArgs pw, GemmArgs pd, int dgrad_blocks) {
   __shared__ float lds[SPLITK_LDS_FLOATS(4)];  // one region for either kind of block
   const int b = blockIdx.x;
   if (b < dgrad_blocks) {
-    splitk_block<true, false, EPI_D, false>(pd, b, 0, lds);
+    splitk_block<true, false, EPI_D, false, 4, PAIR_DEPTH>(pd, b, 0, lds);
   } else {
     const int per = pw.tiles_m * pw.tiles_n, w = b - dgrad_blocks, z = w / per;
-    splitk_block<false, false, EPI_NONE, true>(pw, w - z * per, z, lds);
+    splitk_block<false, false, EPI_NONE, true, 4, PAIR_DEPTH>(pw, w - z * per, z, lds);
   }
 }
 
