@@ -135,46 +135,71 @@ def raw_gemm(args, np, capi):
                       "frac_of_peak": round(tflops / peak, 4)}))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
-    ap.add_argument("--lr", type=float, default=1e-10, help="learning rate (default: the reference benchmark's alpha)")
-    ap.add_argument("--restore-each-step", action="store_true",
-                    help="start every step from the initial weights (a device copy inside the timed region): "
-                         "keeps a loop at a visible learning rate such as 0.01 finite")
-    ap.add_argument("--seed", type=int, default=1)
-    ap.add_argument("--flat-update", action="store_true",
-                    help="one update launch at the end of the step instead of per-layer updates on the second stream")
-    ap.add_argument("--hvariant", type=int, default=0, help="tuning: forced bf16 GEMM tile variant")
-    ap.add_argument("--variants", default="", help="tuning: forced GEMM tile variants 'nt,nn,tn'")
-    ap.add_argument("--serial-backward", action="store_true", help="whole backward pass on one stream")
-    ap.add_argument("--no-graph", action="store_true", help="tuning: every step launched eagerly instead of replaying its graph")
-    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg (0 = skip)")
-    ap.add_argument("--gemm", default="", metavar="M,N,K",
-                    help="instead of the training step: time the forward-type GEMM entry point alone (mi_hgemm_nt / "
-                         "mi_sgemm_nt, dtype of --gemm-dtype, dense random operands) and print one JSON line")
-    ap.add_argument("--gemm-dtype", default="bf16", choices=["bf16", "f32"])
-    args = ap.parse_args()
+def raw_update(args, np, capi):
+    """The reduce+SGD entry points alone on one weight matrix [rows x cols] with R gradient copies,
+    K launches between two stream synchronisations (mlp_omp.cc:240-252 is the pass they stand for):
+      fp32        mi_reduce_sgd_raw         reads R gradients + W, writes W                  (R + 2) * 4 bytes per weight
+      fp32+bf16   mi_reduce_sgd_bf16_raw    the same plus the bf16 copy of W                 + 2
+      fp32+bf16+T mi_reduce_sgd_bf16t_raw   the same plus the transposed bf16 copy, tiled    + 2 + 2
+    Comparing the three shows what each extra write stream costs.  lr = 0: the weights stay what
+    they are however many launches run."""
+    import ctypes
 
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on ONE GPU; there is no multi-GPU path (no collectives). "
-              "Run with --gpus 1.", file=sys.stderr)
-        sys.exit(2)
+    rows, cols, R = (int(x) for x in args.update.split(","))
+    n = rows * cols
+    lib = capi.lib()
+    rng = np.random.default_rng(args.seed)
+    W = capi.DeviceBuffer.from_numpy(rng.standard_normal(n, dtype=np.float32))
+    G = capi.DeviceBuffer(R * n * 4)
+    g = rng.standard_normal(n, dtype=np.float32)
+    for r in range(R):
+        capi.check(lib.mi_memcpy_h2d(G.ptr + r * n * 4, g.ctypes.data_as(ctypes.c_void_p), n * 4))
+    W16, W16T = capi.DeviceBuffer(n * 2), capi.DeviceBuffer(n * 2)
+    lr = ctypes.c_float(0.0)
+    kinds = {
+        "fp32": (lambda: lib.mi_reduce_sgd_raw(W.ptr, G.ptr, n, n, R, lr, None), (R + 2) * 4.0),
+        "fp32+bf16": (lambda: lib.mi_reduce_sgd_bf16_raw(W.ptr, W16.ptr, G.ptr, n, n, R, lr, None), (R + 2) * 4.0 + 2),
+        "fp32+bf16+bf16T": (lambda: lib.mi_reduce_sgd_bf16t_raw(W.ptr, W16.ptr, W16T.ptr, G.ptr, rows, cols, n, R, lr, None),
+                            (R + 2) * 4.0 + 4),
+    }
+    out = {"update": f"{rows} x {cols}, R = {R}", "launches": args.steps, "peak_gbps": PEAK_HBM_GBPS, "kernels": {}}
+    for name, (fn, bytes_per_weight) in kinds.items():
+        for _ in range(max(args.warmup, 5)):
+            capi.check(fn())
+        capi.check(lib.mi_stream_sync(None))
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            capi.check(fn())
+        capi.check(lib.mi_stream_sync(None))
+        us = (time.perf_counter() - t0) / args.steps * 1e6
+        gbps = bytes_per_weight * n / us / 1e3
+        out["kernels"][name] = {"us_per_launch": round(us, 1), "bytes_per_launch": bytes_per_weight * n,
+                                "gbps": round(gbps, 1), "frac_of_peak": round(gbps / PEAK_HBM_GBPS, 4)}
+    print(json.dumps(out))
 
-    import numpy as np
 
-    from tbb_test_amd import capi, hostlib
+def other_config_names(args):
+    """--other-configs: 'auto' = every other benchmark configuration when the headline config runs
+    untuned with default schedule flags, 'none' = skip, or a comma-separated list."""
+    if args.other_configs == "none":
+        return []
+    if args.other_configs == "auto":
+        tuned = (args.config != "C2" or args.hvariant or args.variants or args.serial_backward or args.flat_update
+                 or args.no_graph or args.restore_each_step)
+        return [] if tuned else [c for c in ("C1", "C3", "C4", "C5", "ref") if c != args.config]
+    names = [c for c in args.other_configs.split(",") if c]
+    for c in names:
+        if c not in CONFIGS:
+            raise SystemExit(f"bench.py: unknown configuration {c!r} in --other-configs")
+    return names
 
-    if args.gemm:
-        raw_gemm(args, np, capi)
-        return
 
-    nf, B, R, dtype = CONFIGS[args.config]
+def measure_config(config, args, steps, warmup, info, np, capi, hostlib, min_loop_s=0.0, probe=True):
+    """Times one benchmark configuration on a fresh handle and returns the fields of the JSON line.
+    min_loop_s > 0: the timed loop runs at least that long (more steps than `steps` for the models
+    whose step takes microseconds)."""
+    nf, B, R, dtype = CONFIGS[config]
     layers = len(nf) - 1
-    info = capi.device_info()
 
     X, Ws, dY = hostlib.init_problem(nf, B, R, args.seed)
     flags = (0 if args.flat_update else capi.FLAG_PER_LAYER_UPDATE) | (capi.FLAG_SERIAL_BACKWARD if args.serial_backward else 0)
@@ -205,22 +230,29 @@ def main():
         for _ in range(10):
             one_step()
         h.sync()
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         one_step()
     h.sync()
+    if min_loop_s > 0:   # a first short loop sizes the timed one
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one_step()
+        h.sync()
+        per_step = (time.perf_counter() - t0) / steps
+        steps = int(min(max(steps, min_loop_s / max(per_step, 1e-9)), 2000))
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         one_step()
     h.sync()
     elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
+    ms_per_step = elapsed / steps * 1e3
 
     # per-kernel durations: K more steps, from the initial weights again, with a HIP event pair
     # around every launch
     h.restore_weights()
     h.enable_timing(True)
     h.reset_timings()
-    for _ in range(args.steps):
+    for _ in range(steps):
         one_step()
     ms, cnt = h.timings()
     h.enable_timing(False)
@@ -238,11 +270,13 @@ def main():
         r = ctypes.c_double()
         capi.check(capi.lib().mi_probe_mfma_rate(1 if dtype == "bf16" else 0, operands, ctypes.byref(r), None))
         return round(r.value, 1)
-    mfma_only = {"unit": "TFLOP/s", "random_operands": mfma_rate(2), "ones": mfma_rate(1), "zeros": mfma_rate(0),
-                 "how": "loop of independent MFMAs on register operands, no memory traffic, measured right "
-                        "after the steps above (mi_probe_mfma_rate)"}
-    if dtype == "bf16":  # the large GEMMs use 16x16x32 MFMAs (the figures above); the 32x32x16 shape for comparison
-        mfma_only["random_operands_32x32x16"] = mfma_rate(3)
+    mfma_only = None
+    if probe:
+        mfma_only = {"unit": "TFLOP/s", "random_operands": mfma_rate(2), "ones": mfma_rate(1), "zeros": mfma_rate(0),
+                     "how": "loop of independent MFMAs on register operands, no memory traffic, measured right "
+                            "after the steps above (mi_probe_mfma_rate)"}
+        if dtype == "bf16":  # the large GEMMs use 16x16x32 MFMAs (the figures above); the 32x32x16 shape for comparison
+            mfma_only["random_operands_32x32x16"] = mfma_rate(3)
 
     rows = R * B
     # FLOP of the forward / weight-gradient / input-gradient GEMM of layer l: 2 * rows * N_l * N_{l+1}.
@@ -257,7 +291,7 @@ def main():
     gemm_launches = int(cnt[0:3][:, wide].sum())
     gemm_avg_ms = gemm_ms / gemm_launches
     gemm_tflops = flop_per_gemm / (gemm_avg_ms * 1e-3) / 1e12
-    per_phase = {capi.BREAKDOWN_NAMES[i]: float(ms[i].sum() / args.steps) for i in range(4)}
+    per_phase = {capi.BREAKDOWN_NAMES[i]: float(ms[i].sum() / steps) for i in range(4)}
 
     upd_launches = int(cnt[3].sum())
     upd_ms = float(ms[3].sum()) / upd_launches
@@ -268,7 +302,7 @@ def main():
     upd_gbps = upd_bytes / (upd_ms * 1e-3) / 1e9
 
     peak = PEAK_TFLOPS[dtype]
-    traffic, traffic_note = measured_traffic(args.config)
+    traffic, traffic_note = measured_traffic(config)
     schedule = ("weight and input gradient of a layer in one launch, one stream" if sched["paired_backward"]
                 else "weight-gradient GEMMs on a second stream" if sched["dual_streams"] else "backward pass on one stream")
     schedule += ", per-layer update on the second stream" if sched["per_layer_update"] else ", one update launch"
@@ -278,19 +312,23 @@ def main():
         "value": round(gemm_flop_step / (ms_per_step * 1e-3) / 1e12, 3),
         "unit": "TFLOP/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": dtype,
         "data": "synthetic",
-        "config": {"workload": f"{args.config}: {layers} FC layers, widths "
+        "config": {"workload": f"{config}: {layers} FC layers, widths "
                                + (f"{nf[0]} throughout" if len(set(nf)) == 1 else " ".join(str(v) for v in nf))
                                + f", ReLU between layers, batch {B} per replica x {R} replicas, "
                                + ("every step from the initial weights" if args.restore_each_step else "consecutive steps")
-                               + f", lr {args.lr}, seed {args.seed}",
+                               + f", lr {args.lr}, seed {args.seed}"
+                               + ("" if args.restore_each_step else
+                                  " (the reference's loop and its alpha, mlp_omp.cc:609; the loop at the lr = 0.01 of the "
+                                  "benchmark configurations, which needs every step to start from the initial weights to "
+                                  "stay finite, is --lr 0.01 --restore-each-step)"),
                    "schedule": schedule, "device": info["name"], "num_cus": info["num_cus"]},
         "gemm_flop_per_step": gemm_flop_step,
         "phase_ms_per_step": {k: round(v, 4) for k, v in per_phase.items()},
@@ -312,9 +350,112 @@ def main():
                             "traffic": traffic.get("reduce"),
                             "bytes_per_launch": upd_bytes, "avg_launch_us": round(upd_ms * 1e3, 2)},
     }
+    if sched["paired_backward"]:
+        # the timed loop ran gemm_f32_splitk_pair (weight and input gradient of a layer in one launch);
+        # the event-timed pass keeps separate launches so that every phase has a figure of its own
+        out["roofline"]["note"] = ("phase_ms_per_step, gemm_tflops and this object time the separate weight-gradient and "
+                                   "input-gradient launches (gemm_f32_splitk); ms_per_step and value come from the loop "
+                                   "that runs them paired in one launch per layer")
+    return out
+
+
+def alive_at_exit():
+    """One line on stderr about what this process still holds when it is about to exit: threads
+    other than the main one and child processes (the OpenMP pool of the CPU baseline ends with the
+    process; its task-graph arenas are joined in their destructor)."""
+    import threading
+
+    threads = [t.name for t in threading.enumerate() if t is not threading.main_thread()]
+    children = []
+    try:
+        me = os.getpid()
+        for pid in os.listdir("/proc"):
+            if pid.isdigit():
+                try:
+                    fields = open(f"/proc/{pid}/stat").read().rsplit(")", 1)[1].split()
+                    if int(fields[1]) == me:
+                        children.append(int(pid))
+                except (OSError, IndexError, ValueError):
+                    pass
+        native = len(os.listdir(f"/proc/{me}/task"))
+    except OSError:
+        native = -1
+    print(f"bench.py exit: python threads besides main {threads}, native threads {native}, child processes {children}",
+          file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
+    ap.add_argument("--lr", type=float, default=1e-10, help="learning rate (default: the reference benchmark's alpha)")
+    ap.add_argument("--restore-each-step", action="store_true",
+                    help="start every step from the initial weights (a device copy inside the timed region): "
+                         "keeps a loop at a visible learning rate such as 0.01 finite")
+    ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--flat-update", action="store_true",
+                    help="one update launch at the end of the step instead of per-layer updates on the second stream")
+    ap.add_argument("--hvariant", type=int, default=0, help="tuning: forced bf16 GEMM tile variant")
+    ap.add_argument("--variants", default="", help="tuning: forced GEMM tile variants 'nt,nn,tn'")
+    ap.add_argument("--serial-backward", action="store_true", help="whole backward pass on one stream")
+    ap.add_argument("--no-graph", action="store_true", help="tuning: every step launched eagerly instead of replaying its graph")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--gemm", default="", metavar="M,N,K",
+                    help="instead of the training step: time the forward-type GEMM entry point alone (mi_hgemm_nt / "
+                         "mi_sgemm_nt, dtype of --gemm-dtype, dense random operands) and print one JSON line")
+    ap.add_argument("--gemm-dtype", default="bf16", choices=["bf16", "f32"])
+    ap.add_argument("--update", default="", metavar="ROWS,COLS,R",
+                    help="instead of the training step: time the raw reduce+SGD entry points alone on one weight matrix "
+                         "(mi_reduce_sgd_raw, mi_reduce_sgd_bf16_raw, mi_reduce_sgd_bf16t_raw) and print one JSON line")
+    ap.add_argument("--other-configs", default="auto",
+                    help="'auto' (default): after the headline configuration C2 also time C1, C3, C4, C5 and ref with "
+                         "fresh handles and report them under other_configs; 'none'; or a comma-separated list")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; there is no multi-GPU path (no collectives). "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+
+    from tbb_test_amd import capi, hostlib
+
+    if args.gemm:
+        raw_gemm(args, np, capi)
+        return
+    if args.update:
+        raw_update(args, np, capi)
+        return
+
+    info = capi.device_info()
+    out = measure_config(args.config, args, args.steps, args.warmup, info, np, capi, hostlib)
+    others = other_config_names(args)
+    if others:
+        # The other benchmark configurations, each with a fresh handle in this process, after the
+        # headline measurement: short figures only (the headline's fields stay as they are).
+        out["other_configs"] = {}
+        for name in others:
+            try:
+                full = measure_config(name, args, args.steps, args.warmup, info, np, capi, hostlib, min_loop_s=0.2,
+                                      probe=False)
+                out["other_configs"][name] = {
+                    "ms_per_step": full["ms_per_step"], "value": full["value"], "steps": full["steps"],
+                    "gemm_frac": full["roofline"]["frac"], "reduce_frac": full["roofline_reduce"]["frac"],
+                    "gemm_avg_launch_us": full["roofline"]["avg_launch_us"],
+                    "reduce_avg_launch_us": full["roofline_reduce"]["avg_launch_us"],
+                    "dtype": full["dtype"], "schedule": full["config"]["schedule"], "weights_finite": full["weights_finite"]}
+                if "note" in full["roofline"]:
+                    out["other_configs"][name]["note"] = full["roofline"]["note"]
+            except Exception as exc:   # the headline line is printed whatever happens to the extras
+                out["other_configs"][name] = {"error": f"{type(exc).__name__}: {exc}"}
     if args.cpu_seconds > 0:
+        nf, B, R, _ = CONFIGS[args.config]
         out["cpu_baseline"] = cpu_baseline(nf, B, R, args.lr, args.cpu_seconds)
     print(json.dumps(out), flush=True)
+    alive_at_exit()
 
 
 if __name__ == "__main__":

@@ -85,7 +85,8 @@ struct mi_mlp {
   // dZ_l in dz[l % ndz].  *_fused: the producing GEMM wrote the transposed copy in its epilogue.
   std::vector<uint16_t*> dzT;
   std::vector<char> actsT_fused;  // [L]
-  std::vector<char> dzT_fused;  // [ndz]
+  std::vector<char> dzT_fused;  // [ndz]: state of the slot, what op_wgrad decides on
+  std::vector<char> dzT_fused_layer;  // [L]: whether dZ_l^T last came out of a GEMM epilogue (mi_mlp_get_schedule)
   // bf16 only: the per-replica transposed copy of the uploaded dY, made once by mi_mlp_set_dy (the
   // weight gradient of the last layer reads it every step; the rotation buffers get overwritten)
   uint16_t* dyT = nullptr;
@@ -128,6 +129,10 @@ struct mi_mlp {
   hipGraphExec_t graph_exec = nullptr;
   int graph_epoch = 0;  // g_variant_epoch at capture time
   int eager_steps = 0;
+  // g_variant_epoch of the last untimed eager step (-1: none yet).  A capture follows only such a
+  // step: it has launched every kernel of the schedule once, so that the one-time kernel attribute
+  // calls (more than 64 KB of dynamic LDS) are behind us when the capture begins.
+  int warm_epoch = -1;
   // -lr on the device: the update kernels of a step read it from here, so that a captured graph
   // follows a learning-rate schedule without being captured again
   float* neg_lr_dev = nullptr;
@@ -325,6 +330,7 @@ int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
                      (const uint16_t*)mask, h->nf[l], s, g_hvariant, ct, h->B, &wrote, cp, &wrote_cs);
     if (l > 0) {
       h->dzT_fused[(l - 1) % h->ndz] = wrote;
+      h->dzT_fused_layer[l - 1] = wrote;
       h->colpart_valid[(l - 1) % h->ndz] = wrote_cs;
     }
   }
@@ -486,6 +492,7 @@ int op_loss(mi_mlp* h, hipStream_t s) {
                        per_replica, inv_b, h->loss_partials);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e, "loss launch");
+  h->dyT_valid = false;  // dY was rewritten on the device: the transposed copy made at upload is stale
   return ts.finish();
 }
 
@@ -964,6 +971,7 @@ int mi_mlp_create(mi_mlp** out, int L, const int* nfeatures, int batch_per_repli
     for (int l = 0; l < L; ++l) alloc((void**)&h->actsT[l], (size_t)h->MB * h->nf[l] * 2);
     h->dzT.assign(h->ndz, nullptr);
     h->dzT_fused.assign(h->ndz, 0);
+    h->dzT_fused_layer.assign(L, 0);
     for (int i = 0; i < h->ndz; ++i) alloc((void**)&h->dzT[i], (size_t)h->MB * h->maxw() * 2);
     alloc((void**)&h->dyT, (size_t)h->MB * h->nf[L] * 2);
     h->colpart.assign(h->ndz, nullptr);
@@ -1271,17 +1279,22 @@ int mi_reduce_sgd_layer(mi_mlp* h, int l, float lr) {
 int mi_mlp_step(mi_mlp* h, float lr) {
   if (int rc = check_handle(h)) return rc;
   const bool use_graph = !(h->flags & MI_FLAG_NO_GRAPH) && !h->timing;
-  if (!use_graph || h->eager_steps < 1) {
-    // the first step always runs eagerly: it performs the one-time kernel attribute setup,
-    // which must not happen inside a stream capture
+  const int epoch_now = g_variant_epoch.load();
+  if (h->graph_exec && h->graph_epoch != epoch_now) drop_graph(h);
+  if (!use_graph || h->warm_epoch != epoch_now) {
+    // Eager: the first step, every step of a handle without graph or with per-kernel timing on, and
+    // the first untimed step after a change of the forced tile variants.  Such a step performs the
+    // one-time kernel attribute setup of the kernels it launches, which must not happen inside a
+    // stream capture; a timed step launches other kernels (separate launches, one stream) and so
+    // does not count.
     h->eager_steps++;
     if (int rc = ensure_lr(h, lr)) return rc;
-    return enqueue_step(h, lr);
+    if (int rc = enqueue_step(h, lr)) return rc;
+    if (!h->timing) h->warm_epoch = epoch_now;
+    return MI_OK;
   }
   if (int rc = ensure_lr(h, lr)) return rc;
-  if (h->graph_exec && h->graph_epoch != g_variant_epoch.load()) drop_graph(h);
   if (!h->graph_exec) {
-    const int epoch = g_variant_epoch.load();
     hipGraph_t graph = nullptr;
     MI_HIP(hipStreamBeginCapture(h->stream, hipStreamCaptureModeThreadLocal));
     int rc = enqueue_step(h, lr);
@@ -1297,7 +1310,7 @@ int mi_mlp_step(mi_mlp* h, float lr) {
       h->graph_exec = nullptr;
       return hip_fail(e, "hipGraphInstantiate");
     }
-    h->graph_epoch = epoch;
+    h->graph_epoch = epoch_now;
   }
   MI_HIP(hipGraphLaunch(h->graph_exec, h->stream));
   return MI_OK;
@@ -1376,7 +1389,7 @@ int mi_mlp_get_schedule(mi_mlp* h, int* info) {
   int fused = 0;
   if (h->dtype == MI_BF16) {
     for (int l = 1; l < h->L; ++l) fused += h->actsT_fused[l] ? 1 : 0;  // A_l^T written by forward(l-1)
-    for (int l = 0; l + 1 < h->L; ++l) fused += h->dzT_fused[l % h->ndz] ? 1 : 0;  // dZ_l^T written by dgrad(l+1)
+    for (int l = 0; l + 1 < h->L; ++l) fused += h->dzT_fused_layer[l] ? 1 : 0;  // dZ_l^T written by dgrad(l+1)
   }
   info[3] = fused;
   info[4] = h->last_paired ? 1 : 0;

@@ -1261,6 +1261,21 @@ static hipError_t launch_generic(GemmArgs& p, int batch, hipStream_t s) {
 
 static inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 
+// The automatic choice as far as the shape decides it (aligned operands assumed): which tiling a
+// GEMM of M x N x K with `batch` entries gets.  dispatch() and the paired backward launch of small
+// models both ask this one function, so that the paired launch and the separate launches always
+// run the same kernel on the same shape (and so add up in the same order).
+enum AutoTile { AUTO_128, AUTO_128x64, AUTO_SPLITK, AUTO_64, AUTO_GUARDED };
+static AutoTile auto_tile(int M, int N, int K, long long batch) {
+  auto whole = [&](int bm, int bn, int bk) { return K > 0 && M % bm == 0 && N % bn == 0 && K % bk == 0; };
+  const long long tiles128 = (long long)(M / 128) * (N / 128) * batch;
+  if (whole(128, 128, 16) && tiles128 >= 192) return AUTO_128;       // about one 128 x 128 tile per CU or more
+  if (whole(128, 64, 32) && tiles128 * 2 >= 192) return AUTO_128x64;
+  if (whole(32, 32, 32) && (long long)(M / 64) * (N / 64) * batch < 192) return AUTO_SPLITK;  // fewer 64 x 64 tiles than CUs
+  if (whole(64, 64, 16)) return AUTO_64;
+  return AUTO_GUARDED;
+}
+
 // Picks a tile configuration.  `variant` (0 = automatic) lets the tuning harness force one.
 // `fused_colsum` reports whether the chosen kernel also produced p.colsum.
 template <bool AK, bool BKM, int EPI, bool COLSUM = false>
@@ -1291,9 +1306,9 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
     //     7.90 -> 7.76 ms.)
     // Smaller problems fall back to 128 x 64 and 64 x 64 tiles to get enough workgroups, the
     // smallest (config 1) to the split-K kernel.
-    const long long tiles128 = (long long)(p.M / 128) * (p.N / 128) * batch;
     constexpr bool kWeightGradient = !AK && !BKM;
-    if (fits(128, 128, 16) && tiles128 >= 192) {
+    const AutoTile tile = vec_ok && mask_ok ? auto_tile(p.M, p.N, p.K, batch) : AUTO_GUARDED;
+    if (tile == AUTO_128) {
       variant = 34;
       if (kWeightGradient && p.K < 512) {
         variant = 33;
@@ -1308,12 +1323,12 @@ static hipError_t dispatch(GemmArgs& p, int batch, hipStream_t s, int variant, b
           }
         }
       }
-    } else if (fits(128, 64, 32) && tiles128 * 2 >= 192) {
+    } else if (tile == AUTO_128x64) {
       variant = 11;
-    } else if (fits(32, 32, 32) && (long long)(p.M / 64) * (p.N / 64) * batch < 192) {
+    } else if (tile == AUTO_SPLITK) {
       variant = 50;  // fewer 64 x 64 tiles than CUs: 32 x 32 tiles with K split over the wavefronts
       if (AK && BKM && EPI != EPI_MASK && batch == 1 && p.K % 256 == 0) variant = 51;  // both operands K-contiguous: through the LDS
-    } else if (fits(64, 64, 16)) {
+    } else if (tile == AUTO_64) {
       variant = 16;
     } else if (p.K > 0) {
       // ragged shape or unaligned storage: the guarded MFMA kernels, big tile if it fills the chip
@@ -1403,11 +1418,9 @@ hipError_t sgemm_tn(int R, int M, int N, int K, const float* A, int lda, const f
   return colsum_f32(R, M, K, A, lda, colsum, stride_colsum, s);  // any-shape path: separate kernel
 }
 
-// Whether the automatic choice takes the split-K kernel for a GEMM of this shape (the same rule
-// as in dispatch(): whole 32 x 32 blocks, K a multiple of 32, fewer 64 x 64 tiles than CUs).
+// Whether the automatic choice takes the split-K kernel for a GEMM of this shape.
 static bool splitk_shape(int M, int N, int K, int batch) {
-  return M > 0 && N > 0 && K > 0 && M % 32 == 0 && N % 32 == 0 && K % 32 == 0 &&
-         (long long)(M / 64) * (N / 64) * batch < 192 && (long long)(M / 128) * (N / 128) * batch * 2 < 192;
+  return M > 0 && N > 0 && K > 0 && auto_tile(M, N, K, batch) == AUTO_SPLITK;
 }
 
 bool sgemm_backward_pair_fits(int R, int rows, int nout, int nin) {

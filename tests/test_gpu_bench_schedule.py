@@ -10,7 +10,8 @@ moves the weights visibly).
 Config 2 (the benchmark's headline) runs at full size against the float64-accumulating oracle and,
 bit for bit, against the serial eager schedule.  Config 5 (bf16, 52.8 TFLOP per step) is checked
 through mi_mlp_step on sampled rows for every layer, with the oracle fed the device's own
-operands, and the update of every layer is re-derived bit-exactly from the device's gradients.
+operands (one row per 256-row tile of every output, all replicas of every weight gradient), and the
+update of every layer is re-derived bit-exactly from the device's gradients.
 Bounds: 1e-4 (fp32) / 2e-2 (bf16), norm-wise and element-wise."""
 import numpy as np
 import pytest
@@ -167,18 +168,28 @@ def test_learning_rate_change_needs_no_new_graph_and_is_applied():
     hg.close(); he.close()
 
 
-def test_variant_change_after_capture_is_honoured():
+@pytest.mark.parametrize("variant", [16, 31])
+def test_variant_change_after_capture_is_honoured(variant):
     """A handle that captured its graph re-captures after mi_set_gemm_variant; results keep their
     tolerance and the forced kernel is the one that runs (its bits differ from the automatic one's
-    only through the summation order, so the check is parity, not equality)."""
+    only through the summation order, so the check is parity, not equality).  Variant 16: 64 x 64
+    tiles instead of the split-K kernel.  Variant 31: 128 x 128 x 32 with direct-to-LDS loads, 96 KB
+    of dynamic LDS -- a kernel whose one-time attribute call must not land inside the new capture:
+    the step after the change runs eagerly, the one after that captures."""
     nf, B, R = [512, 512, 512], 256, 2
     h, X, Ws, dY = build(nf, B, R, seed=9, flags=BENCH_FLAGS)
     bench_loop(h, 3)
+    assert h.schedule()["graph"]
     lib = capi.lib()
     try:
         for kind in range(3):
-            capi.check(lib.mi_set_gemm_variant(kind, 16))    # 64 x 64 tiles instead of the split-K kernel
-        bench_loop(h, 2, snapshot=False)
+            capi.check(lib.mi_set_gemm_variant(kind, variant))
+        h.restore_weights()
+        h.step(LR)
+        h.sync()
+        assert not h.schedule()["graph"]      # the old graph is gone, this step ran eagerly
+        bench_loop(h, 3, snapshot=False)
+        assert h.schedule()["graph"]
     finally:
         for kind in range(3):
             lib.mi_set_gemm_variant(kind, 0)
@@ -186,6 +197,36 @@ def test_variant_change_after_capture_is_honoured():
     ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR)
     for l in range(2):
         assert close(h.weight(l), ref.W_new[l], FP32_TOL)
+    h.close()
+
+
+def test_capture_after_a_first_step_under_per_kernel_timing():
+    """A handle whose first steps ran with per-kernel timing on (separate launches on one stream)
+    has not yet launched the kernels of its real schedule; the first untimed step still runs
+    eagerly, the capture comes after it, and replayed steps match the oracle."""
+    nf, B, R = [1024, 1024, 1024], 1024, 4     # large enough for the 84 KB direct-to-LDS kernels on two streams
+    h, X, Ws, dY = build(nf, B, R, seed=4, flags=BENCH_FLAGS)
+    h.snapshot_weights()
+    h.enable_timing(True)
+    for _ in range(2):
+        h.restore_weights()
+        h.step(LR)
+    ms, cnt = h.timings()
+    h.enable_timing(False)
+    assert cnt[:3].sum() == 2 * 3 * 2 and ms[:3].sum() > 0
+    h.restore_weights()
+    h.step(LR)
+    h.sync()
+    assert not h.schedule()["graph"]
+    bench_loop(h, 2, snapshot=False)
+    sched = h.schedule()
+    assert sched["graph"] and sched["dual_streams"] and sched["per_layer_update"]
+    bs = [np.zeros(n, np.float32) for n in nf[1:]]
+    acts = [h.activation(l) for l in range(3)]
+    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR, given_acts=acts)
+    for l in range(2):
+        assert close(h.weight(l), ref.W_new[l], FP32_TOL), f"W {l}"
+    assert close(h.dx(), ref.dX, FP32_TOL)
     h.close()
 
 
@@ -200,9 +241,10 @@ def test_config_5_step_every_layer_on_sampled_rows():
     assert sched["fused_transposes"] == 2 * (L - 1)   # every transposed copy came out of a GEMM epilogue
 
     rng = np.random.default_rng(0)
-    # one batch row in every 256-row tile of the activations, 8 output features per layer
+    # one batch row in every 256-row tile of the activations, and one output feature (= row of dW)
+    # in every 256-row tile of the weight gradients: whole rows, so every tile of every GEMM is touched
     rows = np.arange(0, MB, 256) + rng.integers(0, 256, MB // 256)
-    ms = np.sort(rng.choice(nf[-1], 8, replace=False))
+    ms = np.arange(0, nf[-1], 256) + rng.integers(0, 256, nf[-1] // 256)
 
     prev = h.activation(0)
     for l in range(L):                       # forward: layer by layer on the device's own input
@@ -225,10 +267,9 @@ def test_config_5_step_every_layer_on_sampled_rows():
             sl = slice(r * B, (r + 1) * B)
             dW = h.wgrad_of(l, r)[ms]
             grads.append(dW)
-            if r in (0, R - 1):
-                want = dz[sl][:, ms].astype(np.float64).T @ a[sl].astype(np.float64)
-                assert close(dW, want, BF16_TOL), f"dW layer {l} replica {r}"
-                assert close(h.bgrad_of(l, r), dz[sl].astype(np.float64).sum(0), BF16_TOL), f"db layer {l} replica {r}"
+            want = dz[sl][:, ms].astype(np.float64).T @ a[sl].astype(np.float64)
+            assert close(dW, want, BF16_TOL), f"dW layer {l} replica {r}"
+            assert close(h.bgrad_of(l, r), dz[sl].astype(np.float64).sum(0), BF16_TOL), f"db layer {l} replica {r}"
         del dz, a, out
         # the update, re-derived bit-exactly from the device's own gradients (fp32 master weights),
         # and both bf16 copies the next step's GEMMs read

@@ -305,6 +305,16 @@ def test_bf16_step_falls_back_to_transpose_launches_when_the_batch_does_not_fit_
         lib.mi_set_hgemm_variant(0)
 
 
+@pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, 0])
+def test_fused_transposes_are_counted_per_layer_when_only_some_layers_allow_them(flags):
+    """Widths 64 100 64 64 64 64: the GEMMs around the 100-wide activation run on the guarded tiles,
+    which write no transposed copy.  A_3^T, A_4^T (forward of layers 2, 3) and dZ_1^T, dZ_2^T, dZ_3^T
+    (input gradient of layers 2, 3, 4) come out of GEMM epilogues, A_1^T, A_2^T and dZ_0^T from
+    transpose launches: 5 fused copies, counted per layer although dZ rotates through 3 buffers
+    (dZ_0 and dZ_3 share one)."""
+    _check_bf16_step([64, 100, 64, 64, 64, 64], 64, 2, flags, seed=41, expect_fused=5)
+
+
 def test_bf16_master_weights_stay_fp32():
     """The update is applied to the fp32 master copy: a step whose update is far below bf16
     resolution still changes the weights."""

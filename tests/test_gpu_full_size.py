@@ -2,14 +2,14 @@
 
 Configs 3 and 4 (fp32) are small enough for the float64-accumulating oracle (a few seconds on the
 host): forward compared directly, backward on the device's own activations (identical ReLU masks),
-bound 1e-4.  Config 5 (bf16, 52.8 TFLOP per step) is out of the oracle's reach, so every operation
+bound 1e-4 norm-wise and element-wise.  Config 5 (bf16, 52.8 TFLOP per step) is out of the oracle's reach, so every operation
 is checked on sampled rows against the oracle fed with the device's own operands, bound 2e-2, and
 the update is re-derived bit-exactly on sampled rows from the device's own gradients."""
 import numpy as np
 import pytest
 
 import oracle
-from conftest import BF16_TOL, FP32_TOL, rel_err
+from conftest import BF16_TOL, FP32_TOL, close, elem_err, rel_err
 from tbb_test_amd import capi, hostlib
 
 pytestmark = pytest.mark.gpu
@@ -42,18 +42,18 @@ def test_fp32_config_full_size(name, nf, B, R):
     ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR)
     flips = 0
     for l in range(L + 1):
-        assert rel_err(acts[l], ref.acts[l]) <= FP32_TOL, f"{name} activation {l}"
+        assert close(acts[l], ref.acts[l], FP32_TOL), f"{name} activation {l}: {rel_err(acts[l], ref.acts[l])}, {elem_err(acts[l], ref.acts[l])}"
         flips += int(np.count_nonzero((acts[l] > 0) != (ref.acts[l] > 0)))
     assert flips < 1000, flips
     del ref
     ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR, given_acts=acts)
-    assert rel_err(h.dx(), ref.dX) <= FP32_TOL
+    assert close(h.dx(), ref.dX, FP32_TOL), "dX"
     for l in range(L):
         for r in range(R):
-            assert rel_err(h.wgrad_of(l, r), ref.dW[r][l]) <= FP32_TOL, (l, r)
-            assert rel_err(h.bgrad_of(l, r), ref.db[r][l]) <= FP32_TOL, (l, r)
-        assert rel_err(h.weight(l), ref.W_new[l]) <= FP32_TOL, l
-        assert rel_err(h.bias(l), ref.b_new[l]) <= FP32_TOL, l
+            assert close(h.wgrad_of(l, r), ref.dW[r][l], FP32_TOL), (l, r)
+            assert close(h.bgrad_of(l, r), ref.db[r][l], FP32_TOL), (l, r)
+        assert close(h.weight(l), ref.W_new[l], FP32_TOL), l
+        assert close(h.bias(l), ref.b_new[l], FP32_TOL), l
     h.close()
 
 
@@ -150,4 +150,110 @@ def test_gemm_size_independent_properties_at_full_size(M, N, K, R):
     d1 = capi.DeviceBuffer.from_numpy(onehot)
     assert np.array_equal(fwd(d1), W[:, picks].T)
     for b in (dA, dW_, ddZ, dA2, ddZ2, out_y, out_dx, out_dw, d1):
+        b.free()
+
+
+def _random_bf16_bits(rng, rows, cols):
+    """Dense random bf16 patterns: random sign, exponent 2^-3 .. 2^2, seven random mantissa bits."""
+    v = rng.integers(0, 1 << 16, (rows, cols), dtype=np.uint16)
+    sign, mant, e = v & 0x8000, v & 0x7F, (v >> 7) % 6
+    return (sign | ((0x7C + e) << 7) | mant).astype(np.uint16)
+
+
+def _widen(bits16):
+    return (np.asarray(bits16, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+@pytest.mark.parametrize("which", ["nt", "nn", "tn"])
+def test_bf16_gemm_size_independent_properties_at_full_size(which):
+    """The bf16 entry points at the GEMM shapes of config 5 -- 16384 x 8192 x 8192 for the forward and
+    the input-gradient GEMM, 4 x (8192 x 8192 x 4096) for the weight gradient: 1024 tiles of 256 x 256
+    per launch, far beyond what the oracle can multiply.  Properties that need no oracle: a second run
+    gives the same bits; doubling an operand (exponent + 1, exact in bf16) doubles every result bit
+    for bit (products and fp32 sums scale exactly, and so does the final rounding to bf16), which a
+    dropped, duplicated or misplaced tile would break; a one-hot operand picks rows of the other
+    operand exactly; the masked kernel writes zero exactly where the mask is not positive."""
+    lib = capi.lib()
+    rng = np.random.default_rng({"nt": 11, "nn": 12, "tn": 13}[which])
+    if which == "tn":
+        R, M, N, K = 4, 8192, 8192, 4096       # dW_r = At_r [M x K] * Bt_r [N x K]^T, fp32 out
+        At, Bt = _random_bf16_bits(rng, R * M, K), _random_bf16_bits(rng, R * N, K)
+        dA, dB = capi.DeviceBuffer.from_numpy(At), capi.DeviceBuffer.from_numpy(Bt)
+        dA2 = capi.DeviceBuffer.from_numpy((At + 0x80).astype(np.uint16))
+        out = capi.DeviceBuffer(R * M * N * 4)
+
+        def run(a):
+            capi.check(lib.mi_hgemm_tn(R, M, N, K, a.ptr, K, M * K, dB.ptr, K, N * K, out.ptr, N, M * N, None))
+            capi.check(lib.mi_stream_sync(None))
+            return out.to_numpy((R, M, N))
+        base = run(dA)
+        assert np.array_equal(base.view(np.uint32), run(dA).view(np.uint32)), "second run"
+        assert np.isfinite(base).all() and np.count_nonzero(base) > 0.99 * base.size
+        doubled = run(dA2)
+        assert np.array_equal((2 * base).view(np.uint32), doubled.view(np.uint32)), "doubled operand"
+        del doubled
+        # a sampled row of every 256-row tile against float64 on the host (exact products, fp32 sums: 1e-5)
+        rows = np.arange(0, M, 256) + rng.integers(0, 256, M // 256)
+        for r in range(R):
+            want = _widen(At[r * M + rows]).astype(np.float64) @ _widen(Bt[r * N:(r + 1) * N]).astype(np.float64).T
+            assert close(base[r][rows], want, 1e-5), f"replica {r}"
+        del base
+        picks = rng.integers(0, K, R * M)
+        onehot = np.zeros((R * M, K), np.uint16)
+        onehot[np.arange(R * M), picks] = 0x3F80     # 1.0
+        d1 = capi.DeviceBuffer.from_numpy(onehot)
+        got = run(d1)
+        for r in range(R):
+            want = _widen(Bt[r * N:(r + 1) * N][:, picks[r * M:(r + 1) * M]]).T
+            assert np.array_equal(got[r], want), f"one-hot rows, replica {r}"
+        for b in (dA, dB, dA2, out, d1):
+            b.free()
+        return
+
+    M, N, K = 16384, 8192, 8192
+    A, Bm = _random_bf16_bits(rng, M, K), _random_bf16_bits(rng, N, K)
+    dA, dB = capi.DeviceBuffer.from_numpy(A), capi.DeviceBuffer.from_numpy(Bm)
+    dA2 = capi.DeviceBuffer.from_numpy((A + 0x80).astype(np.uint16))
+    out = capi.DeviceBuffer(M * N * 2)
+    mask = dmask = None
+    if which == "nn":
+        mask = np.where(rng.integers(0, 2, (M, N), dtype=np.uint8) == 1, np.uint16(0x3F80), np.uint16(0xBF80))   # +1 / -1
+        mask[::7, ::5] = 0                                                                                   # and some zeros
+        dmask = capi.DeviceBuffer.from_numpy(mask)
+
+    def run(a):
+        if which == "nt":
+            capi.check(lib.mi_hgemm_nt(M, N, K, a.ptr, K, dB.ptr, K, out.ptr, N, None, 0, None))
+        else:
+            capi.check(lib.mi_hgemm_nn(M, N, K, a.ptr, K, dB.ptr, K, out.ptr, N, dmask.ptr, N, None))
+        capi.check(lib.mi_stream_sync(None))
+        return out.to_numpy((M, N), np.uint16)
+    base = run(dA)
+    assert np.array_equal(base, run(dA)), "second run"
+    fb = _widen(base)
+    assert np.isfinite(fb).all()
+    if which == "nn":
+        keep = _widen(mask) > 0
+        assert np.all(base[~keep] == 0), "masked entries are +0"
+        assert np.count_nonzero(fb[keep]) > 0.99 * np.count_nonzero(keep)
+    else:
+        assert np.count_nonzero(fb) > 0.99 * fb.size
+    assert np.array_equal(_widen(run(dA2)), 2 * fb), "doubled operand"
+    # one sampled row of every 256-row tile against float64 on the host; bound: one rounding to bf16 (2^-8)
+    rows = np.arange(0, M, 256) + rng.integers(0, 256, M // 256)
+    want = _widen(A[rows]).astype(np.float64) @ _widen(Bm).astype(np.float64).T
+    if which == "nn":
+        want = np.where(keep[rows], want, 0.0)
+    assert close(fb[rows], want, 2.0 ** -8), "sampled rows"
+    del fb, base
+    picks = rng.integers(0, K, M)
+    onehot = np.zeros((M, K), np.uint16)
+    onehot[np.arange(M), picks] = 0x3F80
+    d1 = capi.DeviceBuffer.from_numpy(onehot)
+    got = run(d1)
+    want = np.ascontiguousarray(Bm[:, picks].T)
+    if which == "nn":
+        want = np.where(keep, want, np.uint16(0))
+    assert np.array_equal(got, want), "one-hot rows"
+    for b in (dA, dB, dA2, out, d1) + ((dmask,) if dmask else ()):
         b.free()

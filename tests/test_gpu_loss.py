@@ -137,6 +137,33 @@ def test_loss_mode_bf16_model():
     h.close()
 
 
+def test_bf16_explicit_loss_backward_after_set_dy_refreshes_the_transposed_gradient():
+    """Per-operation use: labels, then an uploaded dY (which leaves loss mode and caches dY^T for the
+    weight gradient of the last layer), then an explicit loss_backward that rewrites dY on the
+    device.  The weight and bias gradient of the last layer must come from the rewritten dY."""
+    nf, B, R = [256, 256, 128], 128, 2
+    L = len(nf) - 1
+    h, (X, Ws, bs, labels) = build(nf, B, R, seed=21, flags=capi.FLAG_NO_GRAPH, dtype=capi.MI_BF16)
+    _, _, _, dY = oracle.make_problem(nf, B, R, 21)
+    h.set_dy(dY)
+    for l in range(L):
+        h.forward(l)
+    h.loss_backward()
+    h.wgrad(L - 1)
+    h.sync()
+    dz = h.dz(L - 1)          # what the loss kernel wrote (bf16 values)
+    dY_ref, _ = oracle.l2_loss(h.activation(L), labels, R)
+    assert rel_err(dz, dY_ref) <= 2.0 ** -8
+    assert rel_err(dz, dY) > 0.5   # nothing like the uploaded gradient
+    a = h.activation(L - 1)
+    for r in range(R):
+        sl = slice(r * B, (r + 1) * B)
+        want = dz[sl].astype(np.float64).T @ a[sl].astype(np.float64)
+        assert rel_err(h.wgrad_of(L - 1, r), want) <= BF16_TOL, f"dW replica {r}"
+        assert rel_err(h.bgrad_of(L - 1, r), dz[sl].astype(np.float64).sum(0)) <= BF16_TOL, f"db replica {r}"
+    h.close()
+
+
 def test_loss_without_labels_is_an_error():
     h = capi.MlpHandle([32, 32], 16, 1)
     with pytest.raises(capi.MiError):
