@@ -45,6 +45,7 @@ CONFIGS = {
     "C5": ([8192] * 9, 4096, 4, "bf16"),
     # the reference's own default model (mlp_bench_common.h:26), four sockets of 1024 rows
     "ref": ([1024] * 7 + [1], 1024, 4, "f32"),
+    "ref16": ([1024] * 7 + [1], 1024, 4, "bf16"),   # the same model on the bf16 path (matrix-vector kernels for 1024 -> 1)
 }
 PEAK_TFLOPS = {"f32": 157.3, "bf16": 2516.6}  # MI355X dense MFMA peaks
 PEAK_HBM_GBPS = 8000.0
@@ -145,31 +146,42 @@ def raw_update(args, np, capi):
     they are however many launches run."""
     import ctypes
 
-    rows, cols, R = (int(x) for x in args.update.split(","))
+    rows, cols, R, *extra = (int(x) for x in args.update.split(","))
     n = rows * cols
+    layers = extra[1] if len(extra) > 1 else 1   # matrices laid out one behind the other, as a model's layers are
+    stride = layers * n + (extra[0] if extra else 0)     # floats between consecutive replicas' gradients
     lib = capi.lib()
     rng = np.random.default_rng(args.seed)
-    W = capi.DeviceBuffer.from_numpy(rng.standard_normal(n, dtype=np.float32))
-    G = capi.DeviceBuffer(R * n * 4)
+    w = rng.standard_normal(n, dtype=np.float32)
     g = rng.standard_normal(n, dtype=np.float32)
-    for r in range(R):
-        capi.check(lib.mi_memcpy_h2d(G.ptr + r * n * 4, g.ctypes.data_as(ctypes.c_void_p), n * 4))
-    W16, W16T = capi.DeviceBuffer(n * 2), capi.DeviceBuffer(n * 2)
+    W, G = capi.DeviceBuffer(layers * n * 4), capi.DeviceBuffer(R * stride * 4)
+    for l in range(layers):
+        capi.check(lib.mi_memcpy_h2d(W.ptr + l * n * 4, w.ctypes.data_as(ctypes.c_void_p), n * 4))
+        for r in range(R):
+            capi.check(lib.mi_memcpy_h2d(G.ptr + (r * stride + l * n) * 4, g.ctypes.data_as(ctypes.c_void_p), n * 4))
+    W16, W16T = capi.DeviceBuffer(layers * n * 2), capi.DeviceBuffer(layers * n * 2)
     lr = ctypes.c_float(0.0)
+    turn = [0]
+
+    def at(buf, elem_bytes):     # the matrix of the current launch inside its arena
+        return buf.ptr + (turn[0] % layers) * n * elem_bytes
+
     kinds = {
-        "fp32": (lambda: lib.mi_reduce_sgd_raw(W.ptr, G.ptr, n, n, R, lr, None), (R + 2) * 4.0),
-        "fp32+bf16": (lambda: lib.mi_reduce_sgd_bf16_raw(W.ptr, W16.ptr, G.ptr, n, n, R, lr, None), (R + 2) * 4.0 + 2),
-        "fp32+bf16+bf16T": (lambda: lib.mi_reduce_sgd_bf16t_raw(W.ptr, W16.ptr, W16T.ptr, G.ptr, rows, cols, n, R, lr, None),
+        "fp32": (lambda: lib.mi_reduce_sgd_raw(at(W, 4), at(G, 4), n, stride, R, lr, None), (R + 2) * 4.0),
+        "fp32+bf16": (lambda: lib.mi_reduce_sgd_bf16_raw(at(W, 4), at(W16, 2), at(G, 4), n, stride, R, lr, None), (R + 2) * 4.0 + 2),
+        "fp32+bf16+bf16T": (lambda: lib.mi_reduce_sgd_bf16t_raw(at(W, 4), at(W16, 2), at(W16T, 2), at(G, 4), rows, cols, stride, R, lr, None),
                             (R + 2) * 4.0 + 4),
     }
-    out = {"update": f"{rows} x {cols}, R = {R}", "launches": args.steps, "peak_gbps": PEAK_HBM_GBPS, "kernels": {}}
+    out = {"update": f"{rows} x {cols}, R = {R}, {layers} matrices taken in turn, replica stride {stride} floats", "launches": args.steps, "peak_gbps": PEAK_HBM_GBPS, "kernels": {}}
     for name, (fn, bytes_per_weight) in kinds.items():
         for _ in range(max(args.warmup, 5)):
             capi.check(fn())
+            turn[0] += 1
         capi.check(lib.mi_stream_sync(None))
         t0 = time.perf_counter()
         for _ in range(args.steps):
             capi.check(fn())
+            turn[0] += 1
         capi.check(lib.mi_stream_sync(None))
         us = (time.perf_counter() - t0) / args.steps * 1e6
         gbps = bytes_per_weight * n / us / 1e3
@@ -406,9 +418,11 @@ def main():
                     help="instead of the training step: time the forward-type GEMM entry point alone (mi_hgemm_nt / "
                          "mi_sgemm_nt, dtype of --gemm-dtype, dense random operands) and print one JSON line")
     ap.add_argument("--gemm-dtype", default="bf16", choices=["bf16", "f32"])
-    ap.add_argument("--update", default="", metavar="ROWS,COLS,R",
+    ap.add_argument("--update", default="", metavar="ROWS,COLS,R[,PAD[,LAYERS]]",
                     help="instead of the training step: time the raw reduce+SGD entry points alone on one weight matrix "
-                         "(mi_reduce_sgd_raw, mi_reduce_sgd_bf16_raw, mi_reduce_sgd_bf16t_raw) and print one JSON line")
+                         "(mi_reduce_sgd_raw, mi_reduce_sgd_bf16_raw, mi_reduce_sgd_bf16t_raw) and print one JSON line; "
+                         "PAD = floats between the end of one replica's gradients and the start of the next (default 0), LAYERS = "
+                         "matrices laid out one behind the other and taken in turn, launch by launch (default 1)")
     ap.add_argument("--other-configs", default="auto",
                     help="'auto' (default): after the headline configuration C2 also time C1, C3, C4, C5 and ref with "
                          "fresh handles and report them under other_configs; 'none'; or a comma-separated list")

@@ -706,6 +706,15 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     return !want_ct || (p.ct_rows % bm == 0 && p.ct_rows % 8 == 0 && al16(p.Ct) && batch == 1);
   };
   auto fits = [&](int bm, int bn, int bk) { return vec_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0; };
+  if (variant == 0 && hgemm_is_skinny(p.M, p.N, p.K)) {
+    // a layer of at most SKINNY_MAX outputs is matrix-vector work (forward: N, weight gradient: M,
+    // input gradient: K); the caller makes the transposed copy and the bias gradient by itself
+    if (wrote_ct) *wrote_ct = false;
+    if (wrote_colsum) *wrote_colsum = false;
+    p.Ct = nullptr;
+    p.colsum_part = nullptr;
+    return launch_skinny(p, batch, EPI, s);
+  }
   if (variant == 0) {
     // 256 x 256 tiles with 8 wavefronts and direct-to-LDS loads once they cover the CUs (whole
     // 128-byte lines per row when K allows BK = 64), else smaller tiles for more workgroups
@@ -722,16 +731,30 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
   auto x32_ok = [&]() {
     const int per16 = EPI == EPH_F32 ? 4 : 8;
     return fits(256, 256, 64) && al16(p.C) && p.ldc % per16 == 0 && p.batchC % per16 == 0 &&
-           (EPI != EPH_MASK || (al16(p.mask) && p.ldmask % 8 == 0));
+           (EPI != EPH_MASK || (al16(p.mask) && p.ldmask % 8 == 0)) &&
+           (EPI != EPH_F32 || (long long)p.M * p.ldc * 4 < (1ll << 32));  // fp32 stores: 32-bit byte offsets within an entry
   };
-  if ((variant == 27 || variant == 28) && !x32_ok()) variant = 19;
+  // Variants of the 16x16x32 kernel: 27 = raised wave priority around the MFMAs (the automatic
+  // choice), 28 = without it; 29 / 30 = 27 with all / pairs of the batch entries of an fp32-result
+  // GEMM (the replicas of a weight gradient) chained in one workgroup.  Chaining is not chosen
+  // automatically: on four replicas of 8192 x 8192 x 4096 one workgroup per replica and tile takes
+  // 1.63 ms, pairs 1.65 ms, all four in one workgroup 1.73 ms -- the tile stores of an entry have
+  // one K step to drain before the next wait has to see them gone (the counter retires loads and
+  // stores in order), the wavefronts stall there for longer than a workgroup turnover costs.
+  const bool x32 = variant >= 27 && variant <= 30;
+  if (x32 && !x32_ok()) variant = 19;
+  p.chain = 1;
+  if (EPI == EPH_F32 && batch > 1) {
+    if (variant == 29) p.chain = batch;
+    else if (variant == 30 && batch % 2 == 0) p.chain = 2;
+  }
   p.vec_a = al16(p.A) && p.lda % 8 == 0 && p.batchA % 8 == 0;
   p.vec_b = al16(p.B) && p.ldb % 8 == 0 && p.batchB % 8 == 0;
   // column-sum partials come from the 256 x 256 direct-load kernels (wavefront tiles of 128 rows) only
-  if (p.colsum_part && !((variant == 13 || variant == 19 || variant == 25 || variant == 27 || variant == 28) && EPI != EPH_F32 && batch == 1 && p.M % 128 == 0)) p.colsum_part = nullptr;
+  if (p.colsum_part && !((variant == 13 || variant == 19 || variant == 25 || (variant >= 27 && variant <= 30)) && EPI != EPH_F32 && batch == 1 && p.M % 128 == 0)) p.colsum_part = nullptr;
   if (wrote_colsum) *wrote_colsum = p.colsum_part != nullptr;
   {  // the tile height decides whether the transposed output is possible; if not, drop it
-    const int bm = (variant == 3 || variant == 17) ? 128 : variant == 5 ? 64 : 256;  // (variants 13, 19, 25, 27, 28: 256)
+    const int bm = (variant == 3 || variant == 17) ? 128 : variant == 5 ? 64 : 256;  // (variants 13, 19, 25, 27 .. 30: 256)
     if (want_ct && (EPI == EPH_F32 || variant == 21 || variant == 22 || !ct_ok(bm))) {
       p.Ct = nullptr;
       if (wrote_ct) *wrote_ct = false;
@@ -745,7 +768,7 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     case 17: if (fits(128, 128, 32)) return launch_dma<128, 128, 32, 2, 2, EPI, 4>(p, batch, s); break;
     case 19: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2, 1>(p, batch, s); break;
     case 25: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2, 0>(p, batch, s); break;
-    case 27: return launch_x32(p, batch, EPI, true, s);
+    case 27: case 29: case 30: return launch_x32(p, batch, EPI, true, s);
     case 28: return launch_x32(p, batch, EPI, false, s);
     case 21: if (p.K > 0) return launch_h<128, 128, 32, 2, 2, EPI, 1, 3, true>(p, batch, s); break;
     case 22: if (p.K > 0) return launch_h<64, 64, 32, 2, 2, EPI, 1, 3, true>(p, batch, s); break;

@@ -42,6 +42,9 @@ struct HGemmArgs {
   // Folded over a replica's row blocks they are the bias gradient of the layer whose dZ this GEMM
   // produces, which saves a separate pass over that dZ.
   float* colsum_part;
+  // fp32 results of the 16x16x32 kernel: consecutive batch entries one workgroup walks as one K loop
+  // (0 or 1: one workgroup per entry and tile)
+  int chain;
 };
 
 __device__ __forceinline__ u16 f2bf(float f) {
@@ -99,6 +102,20 @@ __device__ __forceinline__ void load_to_lds(const u16* uniform_base, unsigned la
                : "memory", "m0");
 }
 
+// The same for callers whose LDS address is wave-uniform by construction (derived from values
+// that went through readfirstlane once): taking it as a scalar operand directly keeps the compiler
+// from parking one copy per load instruction in vector registers for a readfirstlane of its own.
+__device__ __forceinline__ void load_to_lds_uniform(const u16* uniform_base, unsigned lane_byte_offset,
+                                                    unsigned uniform_lds_byte_addr) {
+  const unsigned long long b = reinterpret_cast<unsigned long long>(uniform_base);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b), hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+  const unsigned long long sbase = ((unsigned long long)hi << 32) | lo;
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(uniform_lds_byte_addr), "v"(lane_byte_offset), "s"(sbase)
+               : "memory", "m0");
+}
+
 template <int... S, class F>
 __device__ __forceinline__ void static_for_h_impl(std::integer_sequence<int, S...>, F&& f) {
   (f(std::integral_constant<int, S>{}), ...);
@@ -124,5 +141,10 @@ __device__ __forceinline__ void ring_barrier() {
 // Launches the 256 x 256 x 64 kernel built on v_mfma_f32_16x16x32_bf16 (gemm_bf16_x32.hip); the
 // caller has checked the shape and alignment rules listed there.  epi: an EpilogueH value.
 hipError_t launch_x32(HGemmArgs& p, int batch, int epi, bool prio, hipStream_t s);
+
+// gemv_bf16.hip: the same product when M, N or K is at most SKINNY_MAX, as matrix-vector passes
+// (any alignment, any epilogue; no transposed second output, no column-sum partials).
+bool hgemm_is_skinny(int M, int N, int K);
+hipError_t launch_skinny(HGemmArgs& p, int batch, int epi, hipStream_t s);
 
 }  // namespace mi

@@ -59,19 +59,27 @@ __device__ __forceinline__ int swz_b(int row) { return ((row >> 3) & 3) * 2 + ((
 // the four columns described at the top of the file.
 template <int EPI>
 __device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][PB], int row0, int colw, int lane,
-                                          unsigned char* region) {
+                                          unsigned char* region, int bz) {
   const int l16 = lane & 15, q = lane >> 4;
   if constexpr (EPI == EPH_F32) {
-    float* __restrict__ cf = reinterpret_cast<float*>(p.C) + (size_t)blockIdx.z * p.batchC;
+    // natural B order, see the kernel.  A wave-uniform base (the batch entry's matrix) plus one 32-bit
+    // byte offset per lane that walks down the rows: one register of address state, so that the
+    // store burst between two K steps of the chained instance costs no registers the loop needs
+    // (the launcher checks that a matrix spans less than 4 GB).
+    const char* cbase = reinterpret_cast<const char*>(reinterpret_cast<float*>(p.C) + (size_t)bz * p.batchC);
+    unsigned off = 4u * ((unsigned)(row0 + l16) * (unsigned)p.ldc + (unsigned)(colw + 4 * q));
+    asm volatile("" : "+v"(off));  // derived here, not kept in registers across the K loop
+    const unsigned row_step = 64u * (unsigned)p.ldc;  // 16 rows
 #pragma unroll
     for (int jq = 0; jq < QB; ++jq) {
-      float* dst = cf + (size_t)(row0 + 16 * jq + l16) * p.ldc + colw + 4 * q;  // natural B order, see the kernel
 #pragma unroll
-      for (int ip = 0; ip < PB; ++ip) *reinterpret_cast<f32x4*>(dst + 16 * ip) = acc[jq][ip];
+      for (int ip = 0; ip < PB; ++ip)
+        *reinterpret_cast<f32x4*>(const_cast<char*>(cbase) + off + 64 * ip) = acc[jq][ip];
+      off += row_step;
     }
     return;
   } else {
-    u16* __restrict__ ch = reinterpret_cast<u16*>(p.C) + (size_t)blockIdx.z * p.batchC;
+    u16* __restrict__ ch = reinterpret_cast<u16*>(p.C) + (size_t)bz * p.batchC;
     u32x4 pk[QB][2];  // the rounded results: eight consecutive columns per register quadruple
     // The whole mask of the wavefront's tile is requested before the first result is stored: the
     // counter that a load is waited for with retires loads and stores in order, so a mask load
@@ -192,10 +200,24 @@ __device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][P
   }
 }
 
-template <int EPI, int PRIO>
+// CHAIN = true (fp32 results, i.e. the weight gradient): the batch entries of one launch are the
+// replicas of a layer, all with the same (m, n) tiles.  A workgroup keeps its tile and walks
+// p.chain consecutive entries as one long K loop whose two LDS buffers never drain: at the end of an
+// entry's K range the operand bases jump to the next entry, the accumulators are stored as that
+// entry's tile and cleared, and the loop goes on.  The tile loads of the first step of the next
+// entry were requested before those stores, so the wait in front of that step's barrier leaves
+// exactly the stores outstanding (the counter retires loads and stores in order); they have one K
+// step to drain before the next wait has to see them gone.  Prologue, epilogue and workgroup
+// turnover are paid once per p.chain entries.  Needs K / 64 even and at least 4.
+constexpr int TILE_STORES_F32 = QB * PB;  // 16-byte store instructions per wavefront and tile
+
+template <int EPI, int PRIO, bool CHAIN = false>
 __global__ __launch_bounds__(NW * 64) void gemm_bf16_x32(HGemmArgs p) {
+  static_assert(!CHAIN || EPI == EPH_F32, "chained batch entries: fp32 results only");
   extern __shared__ __attribute__((aligned(16))) u16 smem_x[];
-  const unsigned lds_base = (unsigned)(size_t)((__attribute__((address_space(3))) const void*)smem_x);
+  // (made wave-uniform explicitly: everything derived from it for the tile loads then stays in
+  // scalar registers instead of one vector register per load instruction and buffer)
+  const unsigned lds_base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)((__attribute__((address_space(3))) const void*)smem_x));
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l16 = lane & 15, kg = lane >> 4;
@@ -224,19 +246,30 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_x32(HGemmArgs p) {
     const int row = (j * NW + wave) * RPI + lrow;
     offb[j] = 2u * ((unsigned)row * (unsigned)p.ldb + (unsigned)(pc ^ (NAT ? swz_a(row) : swz_b(row))) * 8u);
   }
-  const u16* a_base = p.A + (size_t)blockIdx.z * p.batchA + (size_t)m0 * p.lda;
-  const u16* b_base = p.B + (size_t)blockIdx.z * p.batchB + (size_t)n0 * p.ldb;
+  int bz = CHAIN ? (int)blockIdx.z * p.chain : (int)blockIdx.z;  // first (or only) batch entry of this workgroup
+  const u16* a_base = p.A + (size_t)bz * p.batchA + (size_t)m0 * p.lda;
+  const u16* b_base = p.B + (size_t)bz * p.batchB + (size_t)n0 * p.ldb;
+  const int steps_per_entry = p.K / BK;
+  int a_left = steps_per_entry, b_left = steps_per_entry;  // CHAIN: tiles still to request from the current entry
   auto issue_a = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < NIA; ++j)
-      load_to_lds(a_base, offa[j], lds_base + 2u * (unsigned)(buf * A_ELEMS + (j * NW + wave) * RPI * BK));
+      load_to_lds_uniform(a_base, offa[j], lds_base + 2u * (unsigned)(buf * A_ELEMS + (j * NW + wave) * RPI * BK));
     a_base += BK;
+    if (CHAIN && --a_left == 0) {  // on to the next entry's first K step
+      a_left = steps_per_entry;
+      a_base += p.batchA - p.K;
+    }
   };
   auto issue_b = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < NIB; ++j)
-      load_to_lds(b_base, offb[j], lds_base + 2u * (unsigned)(2 * A_ELEMS + buf * B_ELEMS + (j * NW + wave) * RPI * BK));
+      load_to_lds_uniform(b_base, offb[j], lds_base + 2u * (unsigned)(2 * A_ELEMS + buf * B_ELEMS + (j * NW + wave) * RPI * BK));
     b_base += BK;
+    if (CHAIN && --b_left == 0) {
+      b_left = steps_per_entry;
+      b_base += p.batchB - p.K;
+    }
   };
 
   // LDS byte addresses of this lane's fragments for K chunk 0 / 1 (block 0, buffer 0); blocks and
@@ -263,14 +296,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_x32(HGemmArgs p) {
   };
 
   f32x4 acc[QB][PB];
+  auto clear_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
-  for (int jq = 0; jq < QB; ++jq)
+    for (int jq = 0; jq < QB; ++jq)
 #pragma unroll
-    for (int ip = 0; ip < PB; ++ip)
+      for (int ip = 0; ip < PB; ++ip)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) acc[jq][ip][r] = 0.0f;
+        for (int r = 0; r < 4; ++r) acc[jq][ip][r] = 0.0f;
+  };
+  clear_acc();
 
-  const int nk = p.K / BK;
+  const int nk = CHAIN ? steps_per_entry * p.chain : steps_per_entry;
+  bool stores_in_flight = false;  // CHAIN: the step before ended with the store burst of an entry
   bf16x8 fq[2][4], fp[2][PB];
   // sub-chunk s of a step: K chunk s / 2, m blocks 4 (s % 2) .. 4 (s % 2) + 3
   auto multiply = [&](int s) __attribute__((always_inline)) {
@@ -319,7 +356,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_x32(HGemmArgs p) {
       multiply(s);
       if (s == 2) {
         __builtin_amdgcn_sched_barrier(0);  // and the MFMAs stay above the barrier
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0) & 0xc07f);  // vmcnt(0) and lgkmcnt(0)
+        // lgkmcnt(0), and the tile of step t+1 must have landed; the stores of an entry that ended
+        // with the step before are younger than its loads and may stay outstanding
+        if (CHAIN && stores_in_flight) __builtin_amdgcn_s_waitcnt(vmcnt_imm(TILE_STORES_F32) & 0xc07f);
+        else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0) & 0xc07f);
         ring_barrier();
         if (steady || t + 2 < nk) issue_a(cur);
       }
@@ -328,31 +368,78 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_x32(HGemmArgs p) {
       }
     }
   };
+  using C0 = std::integral_constant<int, 0>;
+  using C1 = std::integral_constant<int, 1>;
   int t = 0;
-  for (; t + 4 <= nk; t += 2) {
-    step(t, std::integral_constant<int, 0>{}, std::true_type{});
-    step(t + 1, std::integral_constant<int, 1>{}, std::true_type{});
+  if constexpr (CHAIN) {
+    // Per entry: a first pair of steps (the first of them right behind the stores of the entry
+    // before), the pairs in between, and -- all entries but the last -- the store of the finished
+    // tile; the last entry ends with the two steps that request nothing more and leaves through the
+    // epilogue below.  An entry has an even number of steps, at
+    // least four, so every step here but those last two has a tile t+2 to request.
+    for (int e = 0; e < p.chain; ++e) {
+      const bool last_entry = e + 1 == p.chain;
+      step(t, C0{}, std::true_type{});
+      stores_in_flight = false;
+      step(t + 1, C1{}, std::true_type{});
+      t += 2;
+      const int pairs_end = (e + 1) * steps_per_entry - (last_entry ? 2 : 0);
+      for (; t < pairs_end; t += 2) {
+        step(t, C0{}, std::true_type{});
+        step(t + 1, C1{}, std::true_type{});
+      }
+      if (!last_entry) {
+        // fenced on both sides: stores drifting down among the next step's MFMAs would keep the old
+        // sums alive next to the new ones, which the register file has no room for
+        __builtin_amdgcn_sched_barrier(0);
+        store_x32<EPI>(p, acc, m0 + wm0, n0 + wn0, lane, nullptr, bz);
+        __builtin_amdgcn_sched_barrier(0);
+        clear_acc();
+        __builtin_amdgcn_sched_barrier(0);
+        ++bz;
+        stores_in_flight = true;
+      }
+    }
+    step(t, C0{}, std::false_type{});
+    step(t + 1, C1{}, std::false_type{});
+  } else {
+    for (; t + 4 <= nk; t += 2) {
+      step(t, C0{}, std::true_type{});
+      step(t + 1, C1{}, std::true_type{});
+    }
+    static_for_h<3>([&](auto sc) {
+      constexpr int s = decltype(sc)::value;
+      if (t + s < nk) step(t + s, std::integral_constant<int, s % 2>{}, std::false_type{});
+    });
   }
-  static_for_h<3>([&](auto sc) {
-    constexpr int s = decltype(sc)::value;
-    if (t + s < nk) step(t + s, std::integral_constant<int, s % 2>{}, std::false_type{});
-  });
 
   unsigned char* region = nullptr;
   if (EPI != EPH_F32 && p.Ct) {
     __syncthreads();  // every wavefront is done with the operand tiles: the LDS is free for the staging
     region = reinterpret_cast<unsigned char*>(smem_x) + (size_t)wave * STAGE_REGION;
   }
-  store_x32<EPI>(p, acc, m0 + wm0, n0 + wn0, lane, region);
+  store_x32<EPI>(p, acc, m0 + wm0, n0 + wn0, lane, region, bz);
 }
 
 template <int EPI, int PRIO>
 hipError_t launch_one(HGemmArgs& p, int batch, hipStream_t s) {
-  auto kern = gemm_bf16_x32<EPI, PRIO>;
-  static LdsOptIn opt_in;
-  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), LDS_BYTES); e != hipSuccess) return e;
   p.tiles_m = p.M / BM;
   p.tiles_n = p.N / BN;
+  if constexpr (EPI == EPH_F32) {
+    // chained batch entries (p.chain > 1, set by the caller's choice): groups of p.chain entries per workgroup
+    const int steps = p.K / BK;
+    if (p.chain > 1 && batch % p.chain == 0 && steps >= 4 && steps % 2 == 0) {
+      auto kern = gemm_bf16_x32<EPI, PRIO, true>;
+      static LdsOptIn opt_in;
+      if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), LDS_BYTES); e != hipSuccess) return e;
+      launch_kernel(kern, dim3(p.tiles_m * p.tiles_n, 1, batch / p.chain), dim3(NW * 64), LDS_BYTES, s, p);
+      return hipGetLastError();
+    }
+  }
+  p.chain = 1;
+  auto kern = gemm_bf16_x32<EPI, PRIO, false>;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), LDS_BYTES); e != hipSuccess) return e;
   launch_kernel(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(NW * 64), LDS_BYTES, s, p);
   return hipGetLastError();
 }

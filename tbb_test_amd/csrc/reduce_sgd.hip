@@ -82,7 +82,11 @@ __global__ __launch_bounds__(256) void reduce_sgd_vec4(float* __restrict__ W, un
       w4[i] = o;
       if (WRITE_BF16) {
         u16x4 h = {f32_to_bf16_rne(o[0]), f32_to_bf16_rne(o[1]), f32_to_bf16_rne(o[2]), f32_to_bf16_rne(o[3])};
-        reinterpret_cast<u16x4*>(W16)[i] = h;
+        // A second stream of ordinary stores next to W's costs far more than its bytes once the data
+        // exceeds the caches (8192 x 8192, R = 4: 225 us without the bf16 copy, 300 us with it, 241 us
+        // with it stored non-temporally); the bf16 copy is read next by a GEMM of a later step.
+        if (STREAM) __builtin_nontemporal_store(h, reinterpret_cast<u16x4*>(W16) + i);
+        else reinterpret_cast<u16x4*>(W16)[i] = h;
       }
     }
   }
@@ -179,6 +183,12 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
 // tile row (tile_y == rows / TR) stand for the `tail` floats that follow the matrix in the
 // arena (the layer's bias and padding), updated the flat way, so that a layer is one launch.
 // GROUP = passes whose loads are in flight together.
+// STREAM (the layer exceeds the caches): the two bf16 copies are stored non-temporally -- as ordinary
+// stores next to W's they cost far more than their bytes -- and the tiles are walked in bands of 16
+// tile rows, column by column inside a band, so that the workgroups running at the same time write
+// runs of 2 KB of the transposed copy where row-major order gives 128-byte pieces 16 KB apart
+// (8192 x 8192, R = 4: 367 us with ordinary stores, 327 us with non-temporal ones, 288 us with the
+// bands as well = 6.5 TB/s).
 // Algorithmic traffic per weight: (R + 2) * 4 + 2 + 2 bytes.
 template <int R_FIXED, bool STREAM, int TR, int TC, int GROUP>
 __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, unsigned short* __restrict__ W16,
@@ -205,8 +215,16 @@ __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, un
     o[3] = fmaf(neg_lr, sum[3], w[3]);
     return o;
   };
+  const int tiles_y = rows / TR, matrix_tiles = tiles_x * tiles_y;
   for (int t = blockIdx.x; t < total_tiles; t += gridDim.x) {
-    const int tile_x = t % tiles_x, tile_y = t / tiles_x;
+    int tile_x = t % tiles_x, tile_y = t / tiles_x;
+    if (STREAM && t < matrix_tiles) {  // bands of BAND tile rows, walked column by column
+      constexpr int BAND = 16;
+      const int per_band = BAND * tiles_x, band = t / per_band, within = t - band * per_band;
+      const int band_rows = tiles_y - band * BAND < BAND ? tiles_y - band * BAND : BAND;
+      tile_x = within / band_rows;
+      tile_y = band * BAND + within - tile_x * band_rows;
+    }
     if (tile_y * TR >= rows) {  // the floats behind the matrix: bias and padding
       const size_t base = (size_t)rows * cols, nvec = tail / 4;
       for (size_t i = (size_t)tile_x * NT + tid; i < nvec; i += (size_t)tiles_x * NT) {
@@ -251,7 +269,8 @@ __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, un
         const f32x4 o = update4(sum[i], w[i]);
         const u16x4 h = {f32_to_bf16_rne(o[0]), f32_to_bf16_rne(o[1]), f32_to_bf16_rne(o[2]), f32_to_bf16_rne(o[3])};
         *reinterpret_cast<f32x4*>(W + off[i]) = o;
-        *reinterpret_cast<u16x4*>(W16 + off[i]) = h;
+        if (STREAM) __builtin_nontemporal_store(h, reinterpret_cast<u16x4*>(W16 + off[i]));
+        else *reinterpret_cast<u16x4*>(W16 + off[i]) = h;
         tile[row][c4 * 2] = (unsigned)h[0] | ((unsigned)h[1] << 16);
         tile[row][c4 * 2 + 1] = (unsigned)h[2] | ((unsigned)h[3] << 16);
       }
@@ -267,7 +286,9 @@ __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, un
 #pragma unroll
       for (int k = 0; k < 8; ++k) e[k] = (tile[part * 8 + k][c >> 1] >> ((c & 1) * 16)) & 0xffffu;
       const u32x4 v = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
-      *reinterpret_cast<u32x4*>(W16T + (size_t)(c0 + c) * rows + r0 + part * 8) = v;
+      u32x4* dst = reinterpret_cast<u32x4*>(W16T + (size_t)(c0 + c) * rows + r0 + part * 8);
+      if (STREAM) __builtin_nontemporal_store(v, dst);
+      else *dst = v;
     }
     __syncthreads();  // the tile is read out before the next one is written
   }
@@ -286,10 +307,12 @@ hipError_t reduce_sgd_tiled(float* W, uint16_t* W16, uint16_t* W16T, const float
   if (!reduce_sgd_tiled_fits(W, W16, W16T, G, rows, cols, stride, tail, R) || R <= 0) return hipErrorInvalidValue;
   const float neg_lr = -lr;
   const bool stream = (double)(R + 1) * (double)rows * (double)cols * 4.0 > 192e6;  // beyond the Infinity Cache
-  // 64 x 64 tiles; 64 x 256, 128 x 128 and 256 x 64 tiles and non-temporal stores were measured on
-  // 8192 x 8192 layers with R = 4 and change nothing (2.83-2.93 ms for 8 layers, 5.0-5.1 TB/s): the
-  // mix of five read and three write streams is what the memory sustains.
-  const int tiles_x = cols / 64, total_tiles = tiles_x * (rows / 64 + (tail ? 1 : 0));
+  // 64 x 64 tiles.  With non-temporal stores of the bf16 copies and the banded tile order (see the
+  // kernel) 64 x 128 and 128 x 128 tiles are within 2 % of them on 8192 x 8192 layers with R = 4
+  // (282-288 us); 64 x 256, 128 x 64 and 128 x 256 tiles are 5-15 % slower.
+  // streaming regime: 64 x 128 tiles where the width allows
+  const bool wide = stream && cols % 128 == 0;
+  const int tiles_x = cols / (wide ? 128 : 64), total_tiles = tiles_x * (rows / 64 + (tail ? 1 : 0));
   // A launch that runs beside a GEMM on another stream (the per-layer update of a bf16 model under
   // the input-gradient GEMM of the next layer) is one workgroup per CU walking the tiles, with half
   // the loads in flight (65 instead of 120 registers at R = 4): that leaves the registers and the
@@ -313,7 +336,9 @@ hipError_t reduce_sgd_tiled(float* W, uint16_t* W16, uint16_t* W16T, const float
                 R, neg_lr, neg_lr_dev, tiles_x, total_tiles)
 #define MI_LAUNCH_TILE(RF)                     \
   do {                                         \
-    if (lean) MI_LAUNCH_TILE3(RF, true, 64, 64, 2);      \
+    if (lean && wide) MI_LAUNCH_TILE3(RF, true, 64, 128, 2);    \
+    else if (lean) MI_LAUNCH_TILE3(RF, true, 64, 64, 2);        \
+    else if (wide) MI_LAUNCH_TILE3(RF, true, 64, 128, 4);       \
     else if (stream) MI_LAUNCH_TILE3(RF, true, 64, 64, 4);      \
     else MI_LAUNCH_TILE3(RF, false, 64, 64, 4);                 \
   } while (0)

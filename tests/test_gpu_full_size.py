@@ -57,6 +57,58 @@ def test_fp32_config_full_size(name, nf, B, R):
     h.close()
 
 
+def test_bf16_reference_default_model_full_size():
+    """The reference's default model (1024 x 6 -> 1, mlp_bench_common.h:26) as a bf16 model at full
+    size: six 1024-wide layers on the MFMA kernels and the 1024 -> 1 layer on the bf16 matrix-vector
+    kernels, through mi_mlp_step on the benchmarked schedule, against the fp32 oracle (2e-2, norm-wise
+    and element-wise); backward on the device's own activations (identical ReLU masks)."""
+    nf, B, R = [1024] * 7 + [1], 1024, 4
+    L = len(nf) - 1
+    h, X, Ws, dY = build(nf, B, R, seed=7, dtype=capi.MI_BF16, flags=capi.FLAG_PER_LAYER_UPDATE | capi.FLAG_KEEP_GRADIENTS)
+    h.snapshot_weights()
+    for _ in range(2):              # the second step replays the captured graph
+        h.restore_weights()
+        h.step(LR)
+    h.sync()
+    bs = [np.zeros(n, np.float32) for n in nf[1:]]
+    acts = [h.activation(l) for l in range(L + 1)]
+    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR)
+    for l in range(L + 1):   # the free-running chain: norm-wise (rounding to bf16 accumulates from layer to layer)
+        assert rel_err(acts[l], ref.acts[l]) <= BF16_TOL, f"activation {l}"
+    W16 = [_widen(_to_bf16_bits(W)) for W in Ws]   # the bf16 copies the GEMMs multiply with
+    for l in range(L):       # each layer on the device's own operands: both bounds
+        want = oracle.fc_forward(acts[l], W16[l], None, relu=(l < L - 1))
+        assert close(acts[l + 1], want, BF16_TOL), f"forward layer {l}: {rel_err(acts[l + 1], want)}, {elem_err(acts[l + 1], want)}"
+    # backward, the free-running chain (every dZ_l is rounded to bf16 on the way down): norm-wise
+    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, LR, given_acts=acts)
+    assert rel_err(h.dx(), ref.dX) <= BF16_TOL, "dX"
+    for l in range(L):
+        for r in range(R):
+            assert rel_err(h.wgrad_of(l, r), ref.dW[r][l]) <= BF16_TOL, (l, r)
+        assert rel_err(h.weight(l), ref.W_new[l]) <= BF16_TOL, l
+    # ... and every operation on the device's own operands (bf16 activations, gradients and weight
+    # copies; what is left is the order of the fp32 sums and the rounding of the result): both bounds
+    for l in reversed(range(L)):
+        dz, a = h.dz(l), acts[l]
+        out = h.dx() if l == 0 else h.dz(l - 1)
+        want = oracle.fc_dgrad(dz, W16[l], a if l > 0 else None)
+        assert close(out, want, BF16_TOL), f"input gradient layer {l}: {rel_err(out, want)}, {elem_err(out, want)}"
+        grads, dbs = [], []
+        for r in range(R):
+            sl = slice(r * B, (r + 1) * B)
+            dW, db = oracle.fc_wgrad(dz[sl], a[sl])
+            grads.append(h.wgrad_of(l, r))
+            dbs.append(h.bgrad_of(l, r))
+            assert close(grads[-1], dW, BF16_TOL), f"dW layer {l} replica {r}"
+            assert close(dbs[-1], db, BF16_TOL) or nf[l + 1] == 1, f"db layer {l} replica {r}"
+            assert rel_err(dbs[-1], db) <= BF16_TOL, f"db layer {l} replica {r}"
+        want = oracle.reduce_sgd(Ws[l].ravel(), np.stack([g.ravel() for g in grads]), LR).reshape(Ws[l].shape)
+        assert np.array_equal(h.weight(l).view(np.uint32), want.view(np.uint32)), f"updated W {l}: bit-exact from the device's gradients"
+        want = oracle.reduce_sgd(np.zeros(nf[l + 1], np.float32), np.stack(dbs), LR)
+        assert np.array_equal(h.bias(l).view(np.uint32), want.view(np.uint32)), f"updated b {l}"
+    h.close()
+
+
 def test_bf16_config_5_full_size_sampled():
     nf, B, R = [8192] * 9, 4096, 4
     L = len(nf) - 1
@@ -158,6 +210,12 @@ def _random_bf16_bits(rng, rows, cols):
     v = rng.integers(0, 1 << 16, (rows, cols), dtype=np.uint16)
     sign, mant, e = v & 0x8000, v & 0x7F, (v >> 7) % 6
     return (sign | ((0x7C + e) << 7) | mant).astype(np.uint16)
+
+
+def _to_bf16_bits(a):
+    """fp32 -> bf16 bit pattern, round to nearest even (numpy restatement of the device rounding)."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
 def _widen(bits16):
