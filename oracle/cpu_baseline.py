@@ -33,6 +33,11 @@ def lib():
         l.port_mlp_run.restype = _ci
         l.port_mlp_dag_run.argtypes = l.port_mlp_run.argtypes
         l.port_mlp_dag_run.restype = _ci
+        l.port_mlp_run_overlap.argtypes = [_ci, ctypes.POINTER(_ci), _ci, _ci, _ci, _ci, ctypes.c_float, _ci, _vp, _vp, _vp,
+                                           _ci, _ci, _ci, _vp, _vp, _vp, ctypes.POINTER(ctypes.c_double)]
+        l.port_mlp_run_overlap.restype = _ci
+        l.port_comm_threads.argtypes = [_ci]
+        l.port_comm_threads.restype = _ci
         l.port_mlp_dag_comm_tasks.argtypes = [_ci]
         l.port_mlp_dag_comm_tasks.restype = _ci
         l.port_check_all_reduce.argtypes = [_ci, _ci, _ci, _ci]
@@ -79,8 +84,11 @@ def host_cores():
 
 
 def run_port(nf, B, R, T, lr, X, dY, W_flat, warmup, iters, restore=True, relu_last=False, use_blas=True,
-             scheduler="omp"):
+             scheduler="omp", comm_threads=0):
     """One call of a port.  scheduler: "omp" (SPMD loop of mlp_omp) or "dag" (task graph of mlp_tbb).
+    comm_threads ("omp" only): threads per socket that run the all-reduce beside the backward GEMMs
+    (the reference's OVERLAP_ALL_REDUCE schedule); 0 = every thread does both, one after the other;
+    -1 = the reference's table by threads per socket (mlp_bench_common.h:40-48).
     Returns (W_out flat, dX, times_ms[5])."""
     L = len(nf) - 1
     MB = B * R
@@ -92,10 +100,13 @@ def run_port(nf, B, R, T, lr, X, dY, W_flat, warmup, iters, restore=True, relu_l
     times = (ctypes.c_double * 5)()
     arr = (_ci * len(nf))(*nf)
     sgemm = find_sgemm()[0] if use_blas else None
-    fn = {"omp": lib().port_mlp_run, "dag": lib().port_mlp_dag_run}[scheduler]
-    rc = fn(L, arr, B, R, T, lr, int(relu_last), X.ctypes.data_as(_vp), dY.ctypes.data_as(_vp),
-            W_flat.ctypes.data_as(_vp), warmup, iters, int(restore), sgemm,
-            W_out.ctypes.data_as(_vp), dX.ctypes.data_as(_vp), times)
+    tail = (lr, int(relu_last), X.ctypes.data_as(_vp), dY.ctypes.data_as(_vp), W_flat.ctypes.data_as(_vp), warmup, iters,
+            int(restore), sgemm, W_out.ctypes.data_as(_vp), dX.ctypes.data_as(_vp), times)
+    if scheduler == "omp" and comm_threads != 0:
+        rc = lib().port_mlp_run_overlap(L, arr, B, R, T, comm_threads, *tail)
+    else:
+        fn = {"omp": lib().port_mlp_run, "dag": lib().port_mlp_dag_run}[scheduler]
+        rc = fn(L, arr, B, R, T, *tail)
     if rc != 0:
         raise RuntimeError(f"{scheduler} port failed with {rc}")
     return W_out, dX, list(times)
@@ -112,11 +123,12 @@ def run(nf, B, R, lr, budget_s):
     X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed=1)
     W_flat = np.concatenate([np.concatenate([Ws[l].ravel(), bs[l].ravel()]) for l in range(L)])
     flop = 3 * 2.0 * R * B * sum(nf[l] * nf[l + 1] for l in range(L))
-    _, _, t = run_port(nf, B, R, T, lr, X, dY, W_flat, 1, 1)          # warm caches, estimate the step time
+    Tc = lib().port_comm_threads(T)   # the reference's table: communication threads from 5 threads per socket on
+    _, _, t = run_port(nf, B, R, T, lr, X, dY, W_flat, 1, 1, comm_threads=Tc)          # warm caches, estimate the step time
     # two thirds of the budget for the OpenMP restatement (the reported value), one third for the task graph
     est = max(t[4] * 1e-3, 1e-6)
     iters = int(max(1, min(200, (budget_s * 2 / 3 - 2 * est) / est)))
-    _, _, t = run_port(nf, B, R, T, lr, X, dY, W_flat, 1, iters)
+    _, _, t = run_port(nf, B, R, T, lr, X, dY, W_flat, 1, iters, comm_threads=Tc)
     ms = t[4]
     out = {
         "value": round(flop / (ms * 1e-3) / 1e12, 5),
@@ -128,8 +140,11 @@ def run(nf, B, R, lr, budget_s):
                               "wgt_update": round(t[3], 3)},
         "sgemm": find_sgemm()[1],
         "sample": f"{iters} full step(s) of the same workload (same model, batch and seeded inputs), "
-                  f"{R} replicas x {T} threads = {R * T} OpenMP threads on {cores} host cores, restatement of "
-                  "mlp_omp (oracle/mlp_omp_port.c)",
+                  f"{R} replicas x {T} threads = {R * T} OpenMP threads on {cores} host cores, "
+                  + (f"{Tc} of the {T} running the all-reduce beside the backward GEMMs (OVERLAP_ALL_REDUCE), " if Tc else
+                     "all-reduce after the GEMMs of a layer (the reference's table sets no communication thread aside "
+                     "below 5 threads per socket), ")
+                  + "restatement of mlp_omp (oracle/mlp_omp_port.c)",
     }
     # The same figures in the units and wording of the reference's report_timing()
     # (mlp_bench_common.cc:92-149): GF/s per core for the GEMM phases (mlp_omp.cc:492,584,675 count

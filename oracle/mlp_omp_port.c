@@ -15,11 +15,17 @@
  *                    activation (mlp_omp.cc:619-691)
  *   update           ring reduce-scatter + all-gather with the SGD update fused into the first
  *                    all-gather step, flag handshakes between neighbouring sockets
- *                    (mlp_omp.cc:56-295), run by all threads after the input gradient: the
- *                    schedule of the reference with OVERLAP_ALL_REDUCE undefined
- *                    (mlp_omp.cc:724-734).  The overlapped schedule needs >= 5 threads per socket
- *                    to have any communication thread (mlp_bench_common.h:40-48), which the host
- *                    shares of the GPU boxes do not offer.
+ *                    (mlp_omp.cc:56-295).  Two schedules, as in the reference:
+ *                    - all threads run the update of a layer after its input gradient
+ *                      (OVERLAP_ALL_REDUCE undefined, mlp_omp.cc:724-734);
+ *                    - overlapped (OVERLAP_ALL_REDUCE, mlp_omp.cc:519-524,601-615,692-723): the last
+ *                      Tc threads of every socket are communication threads.  While the others
+ *                      compute the weight gradient of layer l they run the all-gather (with the
+ *                      SGD update) of layer l+1, while the others compute the input gradient of
+ *                      layer l they run the reduce-scatter of layer l, and after layer 0 its
+ *                      all-gather.  Tc comes from the reference's table by threads per socket
+ *                      (mlp_bench_common.h:40-48: none below 5 threads, so the 4-thread sockets of
+ *                      a 16-core host run the first schedule, like the reference would).
  * and adds what the benchmark configurations add to the reference: bias, ReLU between layers,
  * the ReLU mask in the backward pass, db = column sums, an explicit upstream gradient dY.
  *
@@ -170,52 +176,81 @@ static span_t thread_span(size_t chunk, size_t per_chunk, size_t per_thread, int
   return s;
 }
 
-/* grads, push, weights: ns stacked replicas of `weight_size` floats each. */
-static void ring_update(ring_ctx* rc, float* weights, float* grads, float* push, size_t weight_size, float alpha,
-                        int sid, int t, int* phase) {
-  const int ns = rc->ns, T = rc->T, tid = sid * T + t;
+/* Threads of a socket set aside for the all-reduce when it overlaps the GEMMs, by threads per
+ * socket (mlp_bench_common.h:40-48). */
+int port_comm_threads(int T) {
+  if (T < 5) return 0;
+  if (T < 10) return 1;
+  if (T < 20) return 2;
+  return 4;
+}
+
+typedef struct {
+  int idx, prev, next;
+  size_t per_chunk, per_thread;
+} ring_plan;
+
+static ring_plan plan_ring(const ring_ctx* rc, size_t weight_size, int sid, int t) {
+  const int ns = rc->ns, T = rc->T;
   int ring[3];
   port_ring_info(ns, sid, t, ring);
-  int idx = ring[0];
-  const int prev = ring[1], next = ring[2];
+  ring_plan p;
+  p.idx = ring[0];
+  p.prev = ring[1];
+  p.next = ring[2];
   /* Deviation from the reference, on purpose.  With fewer than 8 sockets the reference keeps
    * idx_in_ring = sid also for the reversed ring of odd tasks (mlp_bench_common.cc:183-189), but
    * the chunk schedule below needs a position that grows along `next`; the reference's rule only
    * closes the ring for 2 sockets, and its own start-up check would fail for 3..7 sockets with
    * two or more threads per socket.  Count the position along the ring direction instead. */
-  if (ns < 8 && (t % 2)) idx = (ns - sid) % ns;
-  const size_t per_chunk = (weight_size + (size_t)ns * LINE - 1) / ns / LINE * LINE;
-  const size_t per_thread = (per_chunk + (size_t)T * LINE - 1) / T / LINE * LINE;
+  if (ns < 8 && (t % 2)) p.idx = (ns - sid) % ns;
+  p.per_chunk = (weight_size + (size_t)ns * LINE - 1) / ns / LINE * LINE;
+  p.per_thread = (p.per_chunk + (size_t)T * LINE - 1) / T / LINE * LINE;
+  return p;
+}
+
+/* grads, push, weights: ns stacked replicas of `weight_size` floats each; rc->T threads of every
+ * socket take part, t is this thread's index among them. */
+
+/* reduce-scatter (mlp_omp.cc:56-169); the last addition is left to the all-gather's first step */
+static void ring_reduce_scatter(ring_ctx* rc, float* grads, float* push, size_t weight_size, int sid, int t, int* phase) {
+  const int ns = rc->ns, T = rc->T, tid = sid * T + t;
+  const ring_plan p = plan_ring(rc, weight_size, sid, t);
   float* g = grads + (size_t)sid * weight_size;
   float* pb = push + (size_t)sid * weight_size;
-  float* w = weights + (size_t)sid * weight_size;
-  float* pb_next = push + (size_t)next * weight_size;
-  float* w_next = weights + (size_t)next * weight_size;
-  const float neg_alpha = -alpha;
-
-  /* reduce-scatter (mlp_omp.cc:89-146) */
+  float* pb_next = push + (size_t)p.next * weight_size;
   for (int step = 0; step < ns - 1; ++step) {
-    int chunk = (idx - step + ns) % ns;
-    span_t s = thread_span((size_t)chunk, per_chunk, per_thread, t, weight_size);
+    int chunk = (p.idx - step + ns) % ns;
+    span_t s = thread_span((size_t)chunk, p.per_chunk, p.per_thread, t, weight_size);
     memcpy(pb_next + s.begin, g + s.begin, sizeof(float) * (s.end - s.begin));
-    handshake(rc, tid, prev * T + t, phase);
+    handshake(rc, tid, p.prev * T + t, phase);
     int rd = (chunk - 1 + ns) % ns;
-    s = thread_span((size_t)rd, per_chunk, per_thread, t, weight_size);
+    s = thread_span((size_t)rd, p.per_chunk, p.per_thread, t, weight_size);
     if (step < ns - 2) {
 #pragma omp simd
       for (size_t i = s.begin; i < s.end; ++i) g[i] = g[i] + pb[i];
     }
   }
+}
 
-  /* all-gather with the update fused into its first step (mlp_omp.cc:205-271) */
+/* all-gather with the update fused into its first step (mlp_omp.cc:171-295) */
+static void ring_allgather(ring_ctx* rc, float* weights, float* grads, float* push, size_t weight_size, float alpha,
+                           int sid, int t, int* phase) {
+  const int ns = rc->ns, T = rc->T, tid = sid * T + t;
+  const ring_plan p = plan_ring(rc, weight_size, sid, t);
+  float* g = grads + (size_t)sid * weight_size;
+  float* pb = push + (size_t)sid * weight_size;
+  float* w = weights + (size_t)sid * weight_size;
+  float* w_next = weights + (size_t)p.next * weight_size;
+  const float neg_alpha = -alpha;
   if (ns == 1) {
-    span_t s = thread_span(0, per_chunk, per_thread, t, weight_size);
+    span_t s = thread_span(0, p.per_chunk, p.per_thread, t, weight_size);
 #pragma omp simd
     for (size_t i = s.begin; i < s.end; ++i) w[i] = fmaf(neg_alpha, g[i], w[i]);
   }
   for (int step = 0; step < ns - 1; ++step) {
-    int chunk = (idx + 1 - step + ns) % ns;
-    span_t s = thread_span((size_t)chunk, per_chunk, per_thread, t, weight_size);
+    int chunk = (p.idx + 1 - step + ns) % ns;
+    span_t s = thread_span((size_t)chunk, p.per_chunk, p.per_thread, t, weight_size);
     if (step == 0) {
 #pragma omp simd
       for (size_t i = s.begin; i < s.end; ++i) {
@@ -226,8 +261,14 @@ static void ring_update(ring_ctx* rc, float* weights, float* grads, float* push,
     } else {
       memcpy(w_next + s.begin, w + s.begin, sizeof(float) * (s.end - s.begin));
     }
-    handshake(rc, tid, prev * T + t, phase);
+    handshake(rc, tid, p.prev * T + t, phase);
   }
+}
+
+static void ring_update(ring_ctx* rc, float* weights, float* grads, float* push, size_t weight_size, float alpha,
+                        int sid, int t, int* phase) {
+  ring_reduce_scatter(rc, grads, push, weight_size, sid, t, phase);
+  ring_allgather(rc, weights, grads, push, weight_size, alpha, sid, t, phase);
 }
 
 /* The reference's start-up check of the all-reduce (mlp_omp.cc:325-373) on an arbitrary shape:
@@ -291,10 +332,12 @@ static mat_t mat_alloc(int rows, int cols) {
  *   times_ms[5] = average per step of {fwd, wgt_grad, bwd, wgt_update, whole step}.
  * Returns 0, -1 on allocation failure, -2 if OpenMP did not provide R*T threads.
  */
-int port_mlp_run(int L, const int* nf, int B, int R, int T, float lr, int relu_last, const float* X, const float* dY,
-                 const float* W_in, int warmup, int iters, int restore, cblas_sgemm_fn sgemm, float* W_out,
-                 float* dX_out, double* times_ms) {
+static int mlp_run(int L, const int* nf, int B, int R, int T, int Tc, float lr, int relu_last, const float* X,
+                   const float* dY, const float* W_in, int warmup, int iters, int restore, cblas_sgemm_fn sgemm,
+                   float* W_out, float* dX_out, double* times_ms) {
   if (!sgemm) sgemm = port_builtin_sgemm;
+  if (Tc < 0 || Tc >= T) return -3;
+  const int Tg = T - Tc; /* threads of a socket that compute the backward GEMMs */
   const int MB = R * B, nthreads = R * T;
   mat_t* act = (mat_t*)calloc((size_t)L + 2, sizeof(mat_t));
   mat_t *wt = (mat_t*)calloc((size_t)L, sizeof(mat_t)), *gr = (mat_t*)calloc((size_t)L, sizeof(mat_t)),
@@ -312,7 +355,8 @@ int port_mlp_run(int L, const int* nf, int B, int R, int T, float lr, int relu_l
     ok &= (gr[l] = mat_alloc(R * brows[l], nf[l])).d != NULL;
     ok &= (pb[l] = mat_alloc(R * brows[l], nf[l])).d != NULL;
   }
-  ring_ctx rc = {R, T, (_Atomic int*)calloc((size_t)nthreads * 16, sizeof(_Atomic int))};
+  /* the ring is run by all T threads of a socket, or by its Tc communication threads */
+  ring_ctx rc = {R, Tc > 0 ? Tc : T, (_Atomic int*)calloc((size_t)nthreads * 16, sizeof(_Atomic int))};
   if (!ok || !rc.done) return -1;
 
   for (int i = 0; i < MB; ++i) memcpy(act[0].d + (size_t)i * act[0].ld, X + (size_t)i * nf[0], sizeof(float) * nf[0]);
@@ -388,11 +432,11 @@ int port_mlp_run(int L, const int* nf, int B, int R, int T, float lr, int relu_l
         /* backward (mlp_omp.cc:513-736) */
         for (int l = L - 1; l >= 0; --l) {
           double t0 = omp_get_wtime();
-          {
-            /* weight gradient: k split over sockets, (m, n) split inside the socket */
+          if (t < Tg) {
+            /* weight gradient: k split over sockets, (m, n) split over the socket's GEMM threads */
             const int m = nf[l + 1], n = nf[l], k = MB;
             const int kps = ceil_div(k, R), k0 = imin(sid * kps, k), k1 = imin(k0 + kps, k);
-            port_partition_2d_intra(m, n, 0.5, 1, T, t, blk);
+            port_partition_2d_intra(m, n, 0.5, 1, Tg, t, blk);
             const int bm = blk[1] - blk[0], bn = blk[3] - blk[2];
             float* g = gr[l].d + (size_t)sid * brows[l] * gr[l].ld;
             if (bm > 0 && bn > 0)
@@ -408,14 +452,20 @@ int port_mlp_run(int L, const int* nf, int B, int R, int T, float lr, int relu_l
                 for (int j = 0; j < bm; ++j) db[j] += z[j];
               }
             }
+            my_phase[1] += omp_get_wtime() - t0;
+          } else if (l < L - 1) {
+            /* communication thread: all-gather + SGD of the layer above (mlp_omp.cc:601-615); its last
+             * reader, the input gradient of that layer, ended at the barrier before */
+            ring_allgather(&rc, wt[l + 1].d, gr[l + 1].d, pb[l + 1].d, (size_t)brows[l + 1] * wt[l + 1].ld, lr, sid, t - Tg,
+                           &phase);
+            my_phase[3] += omp_get_wtime() - t0;
           }
-          my_phase[1] += omp_get_wtime() - t0;
 #pragma omp barrier
           t0 = omp_get_wtime();
-          {
+          if (t < Tg) {
             /* input gradient, in place over the activation; masked by the ReLU derivative */
             const int n = nf[l], k = nf[l + 1];
-            port_partition_2d(MB, n, 0.5, 0, R, sid, T, t, blk);
+            port_partition_2d(MB, n, 0.5, 0, R, sid, Tg, t, blk);
             const int bm = blk[1] - blk[0], bn = blk[3] - blk[2];
             mat_t* C = &act[l == 0 ? L + 1 : l];
             const float* w = wt[l].d + (size_t)sid * brows[l] * wt[l].ld;
@@ -437,12 +487,21 @@ int port_mlp_run(int L, const int* nf, int B, int R, int T, float lr, int relu_l
                       act[l + 1].ld, w + blk[2], wt[l].ld, 0.0f, C->d + (size_t)blk[0] * C->ld + blk[2], C->ld);
               }
             }
+            my_phase[2] += omp_get_wtime() - t0;
+          } else {
+            /* communication thread: reduce-scatter of this layer's gradients (mlp_omp.cc:692-705) */
+            ring_reduce_scatter(&rc, gr[l].d, pb[l].d, (size_t)brows[l] * wt[l].ld, sid, t - Tg, &phase);
+            my_phase[3] += omp_get_wtime() - t0;
           }
-          my_phase[2] += omp_get_wtime() - t0;
 #pragma omp barrier
           t0 = omp_get_wtime();
-          ring_update(&rc, wt[l].d, gr[l].d, pb[l].d, (size_t)brows[l] * wt[l].ld, lr, sid, t, &phase);
-          my_phase[3] += omp_get_wtime() - t0;
+          if (Tc == 0) {
+            ring_update(&rc, wt[l].d, gr[l].d, pb[l].d, (size_t)brows[l] * wt[l].ld, lr, sid, t, &phase);
+            my_phase[3] += omp_get_wtime() - t0;
+          } else if (l == 0 && t >= Tg) { /* the all-gather nothing is left to overlap with (mlp_omp.cc:709-723) */
+            ring_allgather(&rc, wt[0].d, gr[0].d, pb[0].d, (size_t)brows[0] * wt[0].ld, lr, sid, t - Tg, &phase);
+            my_phase[3] += omp_get_wtime() - t0;
+          }
         }
         /* the forward pass of the next step reads the activations the backward pass overwrote:
          * restore the input rows this thread owns is not needed (act[0] is never written), but
@@ -482,4 +541,19 @@ int port_mlp_run(int L, const int* nf, int B, int R, int T, float lr, int relu_l
   for (int l = 0; l < L; ++l) { free(wt[l].d); free(gr[l].d); free(pb[l].d); }
   free(act); free(wt); free(gr); free(pb); free(brows); free((void*)rc.done);
   return rc_code;
+}
+
+int port_mlp_run(int L, const int* nf, int B, int R, int T, float lr, int relu_last, const float* X, const float* dY,
+                 const float* W_in, int warmup, int iters, int restore, cblas_sgemm_fn sgemm, float* W_out,
+                 float* dX_out, double* times_ms) {
+  return mlp_run(L, nf, B, R, T, 0, lr, relu_last, X, dY, W_in, warmup, iters, restore, sgemm, W_out, dX_out, times_ms);
+}
+
+/* The overlapped schedule with Tc communication threads per socket (Tc < 0: the reference's table).
+ * Returns -3 when Tc leaves no GEMM thread. */
+int port_mlp_run_overlap(int L, const int* nf, int B, int R, int T, int Tc, float lr, int relu_last, const float* X,
+                         const float* dY, const float* W_in, int warmup, int iters, int restore, cblas_sgemm_fn sgemm,
+                         float* W_out, float* dX_out, double* times_ms) {
+  if (Tc < 0) Tc = port_comm_threads(T);
+  return mlp_run(L, nf, B, R, T, Tc, lr, relu_last, X, dY, W_in, warmup, iters, restore, sgemm, W_out, dX_out, times_ms);
 }

@@ -63,6 +63,45 @@ def test_port_step_matches_oracle(nf, B, R, T, relu_last, use_blas):
     assert np.abs(again - want).max() <= 1e-5 * np.abs(want).max()
 
 
+@pytest.mark.parametrize("nf,B,R,T,Tc", [([96, 64, 80, 32], 24, 2, 5, -1),    # the reference's table: 1 of 5 threads
+                                        ([64, 64, 64], 16, 2, 3, 1), ([64, 64, 64], 16, 2, 4, 2),
+                                        ([100, 70, 33, 1], 10, 3, 2, 1), ([48, 48], 8, 1, 3, 1),
+                                        ([64, 48, 64, 32], 20, 4, 2, 1)])
+def test_port_overlapped_schedule_matches_oracle(nf, B, R, T, Tc):
+    """The reference's OVERLAP_ALL_REDUCE schedule (mlp_omp.cc:519-524,601-615,692-723): the last Tc
+    threads of a socket run the all-gather of layer l+1 beside the weight gradient of layer l and the
+    reduce-scatter of layer l beside its input gradient.  Same results as the oracle, also over
+    restored and over consecutive steps."""
+    L = len(nf) - 1
+    X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed=8)
+    rng = np.random.default_rng(2)
+    bs = [(0.1 * rng.standard_normal(b.shape)).astype(np.float32) for b in bs]
+    ref = oracle.mlp_step(nf, B, R, X, dY, Ws, bs, 0.01)
+    flat = np.concatenate([np.concatenate([Ws[l].ravel(), bs[l].ravel()]) for l in range(L)])
+    want = np.concatenate([np.concatenate([ref.W_new[l].ravel(), ref.b_new[l].ravel()]) for l in range(L)])
+    got, dX, times = cb.run_port(nf, B, R, T, 0.01, X, dY, flat, 0, 1, use_blas=False, comm_threads=Tc)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    assert np.abs(dX - ref.dX).max() <= 1e-5 * max(np.abs(ref.dX).max(), 1e-30)
+    assert times[3] > 0 and times[4] > 0
+    again, _, _ = cb.run_port(nf, B, R, T, 0.01, X, dY, flat, 1, 2, restore=True, use_blas=False, comm_threads=Tc)
+    assert np.array_equal(again.view(np.uint32), got.view(np.uint32))
+    # two un-restored steps: the all-gather of a step must have landed before the next forward pass
+    step2 = oracle.mlp_step(nf, B, R, X, dY, ref.W_new, ref.b_new, 0.01)
+    want2 = np.concatenate([np.concatenate([step2.W_new[l].ravel(), step2.b_new[l].ravel()]) for l in range(L)])
+    got2, _, _ = cb.run_port(nf, B, R, T, 0.01, X, dY, flat, 0, 2, restore=False, use_blas=False, comm_threads=Tc)
+    assert np.abs(got2 - want2).max() <= 2e-5 * np.abs(want2).max()
+
+
+def test_overlap_table_and_argument_check():
+    lib = cb.lib()
+    assert [lib.port_comm_threads(T) for T in (1, 4, 5, 9, 10, 19, 20, 28)] == [0, 0, 1, 1, 2, 2, 4, 4]
+    nf, B, R = [32, 32], 8, 2
+    X, Ws, bs, dY = oracle.make_problem(nf, B, R, seed=1)
+    flat = np.concatenate([Ws[0].ravel(), bs[0].ravel()])
+    with pytest.raises(RuntimeError):   # no thread left for the GEMMs
+        cb.run_port(nf, B, R, 2, 0.01, X, dY, flat, 0, 1, use_blas=False, comm_threads=2)
+
+
 # ---- the task-graph restatement (mlp_tbb) -----------------------------------------------------------
 
 @pytest.mark.parametrize("nf,B,R,T,relu_last", [([96, 64, 80, 32], 24, 2, 2, False), ([64, 64, 64], 16, 4, 2, True),
