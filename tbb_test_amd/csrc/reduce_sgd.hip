@@ -82,9 +82,10 @@ __global__ __launch_bounds__(256) void reduce_sgd_vec4(float* __restrict__ W, un
       w4[i] = o;
       if (WRITE_BF16) {
         u16x4 h = {f32_to_bf16_rne(o[0]), f32_to_bf16_rne(o[1]), f32_to_bf16_rne(o[2]), f32_to_bf16_rne(o[3])};
-        // A second stream of ordinary stores next to W's costs far more than its bytes once the data
-        // exceeds the caches (8192 x 8192, R = 4: 225 us without the bf16 copy, 300 us with it, 241 us
-        // with it stored non-temporally); the bf16 copy is read next by a GEMM of a later step.
+        // The bf16 copy is read next by a GEMM of a later step: stored non-temporally it does not push
+        // W out of the Infinity Cache (8192 x 8192, R = 4, one matrix updated over and over: 225 us
+        // without the copy, 300 us with it as ordinary stores, 241 us non-temporal; on cold data, eight
+        // such matrices taken in turn, 268 us without the copy and 289 us with it).
         if (STREAM) __builtin_nontemporal_store(h, reinterpret_cast<u16x4*>(W16) + i);
         else reinterpret_cast<u16x4*>(W16)[i] = h;
       }
@@ -183,12 +184,13 @@ hipError_t reduce_sgd(float* W, uint16_t* W16, const float* G, size_t n, size_t 
 // tile row (tile_y == rows / TR) stand for the `tail` floats that follow the matrix in the
 // arena (the layer's bias and padding), updated the flat way, so that a layer is one launch.
 // GROUP = passes whose loads are in flight together.
-// STREAM (the layer exceeds the caches): the two bf16 copies are stored non-temporally -- as ordinary
-// stores next to W's they cost far more than their bytes -- and the tiles are walked in bands of 16
-// tile rows, column by column inside a band, so that the workgroups running at the same time write
-// runs of 2 KB of the transposed copy where row-major order gives 128-byte pieces 16 KB apart
-// (8192 x 8192, R = 4: 367 us with ordinary stores, 327 us with non-temporal ones, 288 us with the
-// bands as well = 6.5 TB/s).
+// STREAM (the layer exceeds the caches): the two bf16 copies are stored non-temporally and the tiles
+// are walked in bands of 16 tile rows, column by column inside a band, so that the workgroups
+// running at the same time write runs of 2 KB of the transposed copy where row-major order gives
+// 128-byte pieces 16 KB apart.  8192 x 8192, R = 4, on cold data (eight such layers taken in turn,
+// as a step does): 365 us = 5.15 TB/s with 64 x 64 tiles, ordinary stores and row-major order,
+// 333 us = 5.64 TB/s = 0.705 of the HBM peak with 64 x 128 tiles, non-temporal stores and bands;
+// the flat fp32 update of the same matrices (no bf16 copies) reaches 0.75 on the same data.
 // Algorithmic traffic per weight: (R + 2) * 4 + 2 + 2 bytes.
 template <int R_FIXED, bool STREAM, int TR, int TC, int GROUP>
 __global__ __launch_bounds__(256) void reduce_sgd_tile(float* __restrict__ W, unsigned short* __restrict__ W16,
@@ -307,9 +309,11 @@ hipError_t reduce_sgd_tiled(float* W, uint16_t* W16, uint16_t* W16T, const float
   if (!reduce_sgd_tiled_fits(W, W16, W16T, G, rows, cols, stride, tail, R) || R <= 0) return hipErrorInvalidValue;
   const float neg_lr = -lr;
   const bool stream = (double)(R + 1) * (double)rows * (double)cols * 4.0 > 192e6;  // beyond the Infinity Cache
-  // 64 x 64 tiles.  With non-temporal stores of the bf16 copies and the banded tile order (see the
-  // kernel) 64 x 128 and 128 x 128 tiles are within 2 % of them on 8192 x 8192 layers with R = 4
-  // (282-288 us); 64 x 256, 128 x 64 and 128 x 256 tiles are 5-15 % slower.
+  // 64 x 64 tiles in the cached regime.  Streaming regime, cold 8192 x 8192 layers with R = 4 (the
+  // kernel body in a stand-alone loop over four such layers): 64 x 128 tiles in bands 330 us,
+  // 256 x 128 row-major 333 us, 128 x 128 row-major 339 us, 128 x 128 in bands 354 us, 64 x 64 in
+  // bands 361 us, 256 x 64 row-major 376 us, 64 x 64 row-major 380 us, 64 x 64 column-major 467 us;
+  // without the transposed copy 306 us.
   // streaming regime: 64 x 128 tiles where the width allows
   const bool wide = stream && cols % 128 == 0;
   const int tiles_x = cols / (wide ? 128 : 64), total_tiles = tiles_x * (rows / 64 + (tail ? 1 : 0));
