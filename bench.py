@@ -14,6 +14,10 @@ sum-reduced updates stay finite however many steps are run (--lr 0.01 --restore-
 the same step at the learning rate of the parity tests, with a device copy of the weights added
 to every step).
 
+After the headline configuration (--config, default C2) the default run times the other benchmark
+configurations the same way on fresh handles and reports them under other_configs
+(--other-configs none skips them).  --gemm and --update time single entry points instead.
+
 Prints one JSON line:
   value          whole-step throughput, TFLOP/s on the reference's FLOP model
                  3 * 2 * (R*B) * sum_l N_l*N_{l+1}   (mlp_omp.cc:492,584,675)
