@@ -11,7 +11,7 @@ expresses that order with a HIP stream.  Here the caller creates one with hipStr
     W <- W - lr sum_r dW_r         mi_reduce_sgd_raw
 
 twice in a row on it with no host synchronisation in between -- every operation reads what the one
-before wrote, and the second round reads the W the first round updated -- then waits with
+before wrote, and the second pass reads the W the first pass updated -- then waits with
 mi_stream_sync(stream) and compares with the CPU oracle run in the same order.  Bounds: 1e-4 on Y
 and dW, the update bit-exact from the device's own gradients."""
 import ctypes
@@ -61,15 +61,15 @@ def test_chain_of_raw_operations_on_a_caller_stream(B, R, K, N):
     # every buffer is filled by a host-synchronous upload: nothing of the set-up is still in flight
     # on another stream when the caller's stream starts
     dY, dG, dS = _dev(np.zeros(M * N)), _dev(np.zeros(R * stride)), _dev(np.zeros(R * N))
-    # the first round's results are kept by device copies on the same stream (the update kernel with
+    # the first pass's results are kept by device copies on the same stream (the update kernel with
     # one replica and lr = -1 adds its source to a zeroed destination: dst = fma(1, src, 0) = src)
     keep = [(_dev(np.zeros(M * N)), dY, M * N), (_dev(np.zeros(R * stride)), dG, R * stride), (_dev(np.zeros(N * K)), dW, N * K)]
     try:
-        for rnd in range(2):
+        for turn in range(2):
             capi.check(lib.mi_sgemm_nt(M, N, K, dX.ptr, K, dW.ptr, K, dY.ptr, N, db.ptr, 1, stream))
             capi.check(lib.mi_sgemm_tn(R, N, K, B, dY.ptr, N, dX.ptr, K, dG.ptr, K, stride, dS.ptr, N, stream))
             capi.check(lib.mi_reduce_sgd_raw(dW.ptr, dG.ptr, N * K, stride, R, ctypes.c_float(LR), stream))
-            if rnd == 0:
+            if turn == 0:
                 for dst, src, n in keep:
                     capi.check(lib.mi_reduce_sgd_raw(dst.ptr, src.ptr, n, n, 1, ctypes.c_float(-1.0), stream))
         capi.check(lib.mi_stream_sync(stream))
@@ -84,7 +84,7 @@ def test_chain_of_raw_operations_on_a_caller_stream(B, R, K, N):
     finally:
         rt.hipStreamDestroy(stream)
 
-    # round 1 from W0, round 2 from the device's own W after round 1 (so that each round is held to 1e-4 by itself)
+    # first pass from W0, second pass from the device's own W after the first (so that each pass is held to 1e-4 by itself)
     for Wstart, y, g, w in ((W0, y1, g1, w1), (w1, y2, g2, w2)):
         Y = oracle.fc_forward(X, Wstart, b, relu=True)
         assert close(y, Y, FP32_TOL), "forward output"
