@@ -716,12 +716,17 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     return launch_skinny(p, batch, EPI, s);
   }
   if (variant == 0) {
-    // 256 x 256 tiles with 8 wavefronts and direct-to-LDS loads once they cover the CUs (whole
-    // 128-byte lines per row when K allows BK = 64), else smaller tiles for more workgroups
+    // 256 x 256 tiles with 8 wavefronts and direct-to-LDS loads (whole 128-byte lines per row when
+    // K allows BK = 64) from somewhat more than half a round of the 256 CUs on, else 128 x 128 tiles
+    // with direct loads, two workgroups per CU.  One box, forward entry point, us per launch with
+    // 256 x 256 x 64 / 128 x 128 x 32 direct / 128 x 128 x 32 through registers:
+    //   8192 x 1536 x 1536 (192 big tiles) 45.1 / 61.5 / 68.4    4096 x 2048 x 2048 (128) 50.1 / 48.2 / 47.9
+    //   4096 x 1024 x 1024 (64) 25.4 / 12.2 / 16.5               2048 x 2048 x 2048 (64) 43.5 / 23.4 / 33.4
+    //   4096 x 1024 x 4096 (64) 77.1 / 45.1 / 64.4               2048 x 1024 x 1024 (32) 24.2 / 10.2 / 15.1
     const long long t256 = (long long)(p.M / 256) * (p.N / 256) * batch;
-    if (fits(256, 256, 64) && t256 >= 256) variant = 27;  // falls back to 19 below if C or the mask is not 16-byte aligned
+    if (fits(256, 256, 64) && t256 >= 144) variant = 27;  // falls back to 19 below if C or the mask is not 16-byte aligned
     else if (fits(256, 256, 32) && t256 >= 256) variant = 13;
-    else if (fits(128, 128, 32) && (long long)(p.M / 128) * (p.N / 128) * batch >= 128) variant = 3;
+    else if (fits(128, 128, 32) && (long long)(p.M / 128) * (p.N / 128) * batch >= 128) variant = 17;
     else if (fits(64, 64, 32)) variant = 5;
     else if (p.K > 0)  // ragged shape or unaligned storage: the guarded MFMA instances
       variant = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * batch >= 192 ? 21 : 22;

@@ -1269,7 +1269,11 @@ enum AutoTile { AUTO_128, AUTO_128x64, AUTO_SPLITK, AUTO_64, AUTO_GUARDED };
 static AutoTile auto_tile(int M, int N, int K, long long batch) {
   auto whole = [&](int bm, int bn, int bk) { return K > 0 && M % bm == 0 && N % bn == 0 && K % bk == 0; };
   const long long tiles128 = (long long)(M / 128) * (N / 128) * batch;
-  if (whole(128, 128, 16) && tiles128 >= 192) return AUTO_128;       // about one 128 x 128 tile per CU or more
+  // More than 128 big tiles: 128 x 128, one workgroup per CU.  Half tiles would then number more than
+  // the 256 CUs, and the CUs that get two of them decide the launch (1536 x 1536 x 1536, 144 big
+  // tiles: 95.7 us on 128 x 128, 120.8 us on 128 x 64; 3072 x 1024 x 1024: 70.7 / 85.3 us).  Up to 128
+  // big tiles the half tiles still have a CU each (2048 x 1024 x 1024: 64.8 / 47.0 us).
+  if (whole(128, 128, 16) && tiles128 > 128) return AUTO_128;
   if (whole(128, 64, 32) && tiles128 * 2 >= 192) return AUTO_128x64;
   if (whole(32, 32, 32) && (long long)(M / 64) * (N / 64) * batch < 192) return AUTO_SPLITK;  // fewer 64 x 64 tiles than CUs
   if (whole(64, 64, 16)) return AUTO_64;
