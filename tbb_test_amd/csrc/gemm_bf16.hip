@@ -718,15 +718,21 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
   if (variant == 0) {
     // 256 x 256 tiles with 8 wavefronts and direct-to-LDS loads (whole 128-byte lines per row when
     // K allows BK = 64) from somewhat more than half a round of the 256 CUs on, else 128 x 128 tiles
-    // with direct loads, two workgroups per CU.  One box, forward entry point, us per launch with
-    // 256 x 256 x 64 / 128 x 128 x 32 direct / 128 x 128 x 32 through registers:
-    //   8192 x 1536 x 1536 (192 big tiles) 45.1 / 61.5 / 68.4    4096 x 2048 x 2048 (128) 50.1 / 48.2 / 47.9
-    //   4096 x 1024 x 1024 (64) 25.4 / 12.2 / 16.5               2048 x 2048 x 2048 (64) 43.5 / 23.4 / 33.4
-    //   4096 x 1024 x 4096 (64) 77.1 / 45.1 / 64.4               2048 x 1024 x 1024 (32) 24.2 / 10.2 / 15.1
+    // with direct loads, two workgroups per CU: with more than one tile per CU eight wavefronts on
+    // two buffers of BK = 64 (variant 18), else four wavefronts on a ring of four of BK = 32
+    // (variant 17).  One box, forward entry point, us per launch with 256 x 256 x 64 / variant 18 /
+    // variant 17 / 128 x 128 x 32 through registers (variant 3), number of 256 x 256 tiles in brackets:
+    //   8192 x 1536 x 1536 (192) 45.7 / 48.0 / 60.1 / 68.4    6144 x 2048 x 1024 (192) 31.8 / 32.4 / 37.2 / -
+    //   4096 x 2048 x 2048 (128) 50.1 / 38.6 / 50.5 / 47.9    4096 x 2048 x  512 (128) 19.5 / 13.2 / 14.9 / -
+    //   3072 x 2048 x 2048  (96) 45.6 / 32.2 / 40.7 / -       4096 x 1536 x 1536  (96) 37.2 / 25.0 / 32.9 / -
+    //   2048 x 2048 x 2048  (64) 43.5 / 25.0 / 23.0 / 33.4    4096 x 1024 x 4096  (64) 77.1 / 48.6 / 46.4 / 64.4
+    //   4096 x 1024 x 1024  (64) 25.4 / 12.1 / 12.3 / 16.5    2048 x 1024 x 1024  (32) 24.2 / 10.0 / 10.2 / 15.1
     const long long t256 = (long long)(p.M / 256) * (p.N / 256) * batch;
+    const long long t128 = (long long)(p.M / 128) * (p.N / 128) * batch;
     if (fits(256, 256, 64) && t256 >= 144) variant = 27;  // falls back to 19 below if C or the mask is not 16-byte aligned
     else if (fits(256, 256, 32) && t256 >= 256) variant = 13;
-    else if (fits(128, 128, 32) && (long long)(p.M / 128) * (p.N / 128) * batch >= 128) variant = 17;
+    else if (fits(128, 128, 64) && t128 > 256) variant = 18;
+    else if (fits(128, 128, 32) && t128 >= 128) variant = 17;
     else if (fits(64, 64, 32)) variant = 5;
     else if (p.K > 0)  // ragged shape or unaligned storage: the guarded MFMA instances
       variant = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * batch >= 192 ? 21 : 22;
@@ -759,7 +765,7 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
   if (p.colsum_part && !((variant == 13 || variant == 19 || variant == 25 || (variant >= 27 && variant <= 30)) && EPI != EPH_F32 && batch == 1 && p.M % 128 == 0)) p.colsum_part = nullptr;
   if (wrote_colsum) *wrote_colsum = p.colsum_part != nullptr;
   {  // the tile height decides whether the transposed output is possible; if not, drop it
-    const int bm = (variant == 3 || variant == 17) ? 128 : variant == 5 ? 64 : 256;  // (variants 13, 19, 25, 27 .. 30: 256)
+    const int bm = (variant == 3 || variant == 17 || variant == 18) ? 128 : variant == 5 ? 64 : 256;  // (variants 13, 19, 25, 27 .. 30: 256)
     if (want_ct && (EPI == EPH_F32 || variant == 21 || variant == 22 || !ct_ok(bm))) {
       p.Ct = nullptr;
       if (wrote_ct) *wrote_ct = false;
@@ -771,6 +777,7 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     case 5: if (fits(64, 64, 32)) return launch_h<64, 64, 32, 2, 2, EPI>(p, batch, s); break;
     case 13: if (fits(256, 256, 32)) return launch_dma<256, 256, 32, 2, 4, EPI, 4>(p, batch, s); break;
     case 17: if (fits(128, 128, 32)) return launch_dma<128, 128, 32, 2, 2, EPI, 4>(p, batch, s); break;
+    case 18: if (fits(128, 128, 64)) return launch_dma<128, 128, 64, 2, 4, EPI, 2, 1>(p, batch, s); break;
     case 19: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2, 1>(p, batch, s); break;
     case 25: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2, 0>(p, batch, s); break;
     case 27: case 29: case 30: return launch_x32(p, batch, EPI, true, s);

@@ -58,7 +58,7 @@ HSHAPES = [(64, 64, 32), (128, 128, 64), (256, 256, 96), (512, 256, 128), (256, 
            (256, 256, 64), (256, 256, 192), (256, 256, 320), (256, 256, 448),
            # twelve 256 x 256 tiles, three K steps
            (1024, 768, 192)]
-HVARIANTS = [0, 3, 4, 5, 13, 17, 19, 21, 22, 25, 27, 28, 29, 30]
+HVARIANTS = [0, 3, 4, 5, 13, 17, 18, 19, 21, 22, 25, 27, 28, 29, 30]
 # 21, 22: guarded any-shape MFMA instances; 25: 19 without wave priorities; 27, 28: 16x16x32 MFMAs;
 # 29 / 30: 27 with all / pairs of the batch entries of a weight gradient chained in one workgroup
 
@@ -413,7 +413,7 @@ def test_bf16_step_matches_fp32_oracle(name, flags):
     _check_bf16_step(nf, B, R, flags)
 
 
-@pytest.mark.parametrize("variant", [13, 17, 19, 25, 27, 28])
+@pytest.mark.parametrize("variant", [13, 17, 18, 19, 25, 27, 28])
 @pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, 0])
 def test_bf16_step_on_the_large_tile_kernels(variant, flags):
     """The direct-load kernels (256 x 256 and 128 x 128 tiles), which small models never pick by
