@@ -115,14 +115,67 @@ __global__ __launch_bounds__(256) void gemv_bf16_shortk_kernel(HGemmArgs p) {
   }
 }
 
+// The same with 8 consecutive columns of one row per thread: 16-byte accesses to C (two for fp32
+// results) and to the mask.  The sums run over k in the same order as in the kernel above, so both
+// give the same bits.  For N a multiple of 8 and 16-byte aligned rows of C and of the mask.
+template <int EPI>
+__global__ __launch_bounds__(256) void gemv_bf16_shortk_vec_kernel(HGemmArgs p) {
+  const int z = blockIdx.y;
+  const u16* A = p.A + (size_t)z * p.batchA;
+  const u16* B = p.B + (size_t)z * p.batchB;
+  const unsigned groups = (unsigned)p.N >> 3, total = (unsigned)p.M * groups;  // the launcher checks that this fits 32 bits
+  for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+    const unsigned row = i / groups, col = (i - row * groups) * 8u;
+    const u16* a = A + (size_t)row * p.lda;
+    float v[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) v[c] = 0.0f;
+    for (int k = 0; k < p.K; ++k) {
+      const float av = bf2f(a[k]);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) v[c] = fmaf(av, bf2f(B[(size_t)(col + c) * p.ldb + k]), v[c]);
+    }
+    if (EPI == EPH_F32) {
+      float* out = reinterpret_cast<float*>(p.C) + (size_t)z * p.batchC + (size_t)row * p.ldc + col;
+      typedef float f32x4 __attribute__((ext_vector_type(4)));
+      *reinterpret_cast<f32x4*>(out) = f32x4{v[0], v[1], v[2], v[3]};
+      *reinterpret_cast<f32x4*>(out + 4) = f32x4{v[4], v[5], v[6], v[7]};
+      continue;
+    }
+    if (EPI == EPH_BIAS_RELU) {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        if (p.bias) v[c] += p.bias[col + c];
+        if (p.relu) v[c] = v[c] > 0.0f ? v[c] : 0.0f;
+      }
+    } else if (EPI == EPH_MASK) {
+      const u32x4 m = *reinterpret_cast<const u32x4*>(p.mask + (size_t)row * p.ldmask + col);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (!(lo16(m[e]) > 0.0f)) v[2 * e] = 0.0f;
+        if (!(hi16(m[e]) > 0.0f)) v[2 * e + 1] = 0.0f;
+      }
+    }
+    u32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (unsigned)f2bf(v[2 * e]) | ((unsigned)f2bf(v[2 * e + 1]) << 16);
+    *reinterpret_cast<u32x4*>(reinterpret_cast<u16*>(p.C) + (size_t)z * p.batchC + (size_t)row * p.ldc + col) = o;
+  }
+}
+
 template <int EPI>
 hipError_t launch_skinny_epi(HGemmArgs& p, int batch, hipStream_t s) {
   auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   const bool vec = al16(p.A) && al16(p.B) && p.lda % 8 == 0 && p.ldb % 8 == 0 && p.batchA % 8 == 0 && p.batchB % 8 == 0;
   if (p.K <= SKINNY_MAX) {
-    size_t blocks = ((size_t)p.M * p.N + 255) / 256;
+    const int per16 = EPI == EPH_F32 ? 4 : 8;  // elements of C in 16 bytes
+    const bool wide = p.N % 8 == 0 && al16(p.C) && p.ldc % per16 == 0 && p.batchC % per16 == 0 &&
+                      (EPI != EPH_MASK || (al16(p.mask) && p.ldmask % 8 == 0)) &&
+                      (size_t)p.M * (size_t)(p.N / 8) <= 0xffffffffu - 16384u * 256u;
+    size_t blocks = ((size_t)p.M * (wide ? p.N / 8 : p.N) + 255) / 256;
     if (blocks > 16384) blocks = 16384;
-    launch_kernel(gemv_bf16_shortk_kernel<EPI>, dim3((unsigned)blocks, batch), dim3(256), 0, s, p);
+    if (wide) launch_kernel(gemv_bf16_shortk_vec_kernel<EPI>, dim3((unsigned)blocks, batch), dim3(256), 0, s, p);
+    else launch_kernel(gemv_bf16_shortk_kernel<EPI>, dim3((unsigned)blocks, batch), dim3(256), 0, s, p);
   } else if (p.N <= SKINNY_MAX) {
     const dim3 grid((p.M + 3) / 4, batch);
     if (vec) launch_kernel((gemv_bf16_rows_kernel<EPI, true, true>), grid, dim3(256), 0, s, p);

@@ -123,23 +123,25 @@ def test_hgemm_skinny_shapes_all_entry_points(shape):
     assert rel_err(got, oracle.fc_dgrad(A, np.ascontiguousarray(B.T), act)) <= 4e-3, shape
     assert np.all(got[act <= 0] == 0.0)
     # weight-gradient form: R batch entries, fp32 results, entries and results not back to back
+    # (result stride: once odd, once a multiple of 16 bytes, which allows vector stores)
     R = 3
-    sa, sb, sc = M * K + 8, N * K + 16, M * N + 5
+    sa, sb = M * K + 8, N * K + 16
     At = np.zeros((R, sa), np.float32)
     Bt = np.zeros((R, sb), np.float32)
     for r in range(R):
         At[r, :M * K] = bf16_round(rng.standard_normal(M * K))
         Bt[r, :N * K] = bf16_round(rng.uniform(-1, 1, N * K))
     dAt, dBt = dev16(At), dev16(Bt)
-    dW = capi.DeviceBuffer(R * sc * 4)
-    dW.zero()
-    capi.check(lib.mi_hgemm_tn(R, M, N, K, dAt.ptr, K, sa, dBt.ptr, K, sb, dW.ptr, N, sc, None))
-    capi.check(lib.mi_stream_sync(None))
-    out = dW.to_numpy((R, sc))
-    for r in range(R):
-        want = At[r, :M * K].reshape(M, K).astype(np.float64) @ Bt[r, :N * K].reshape(N, K).astype(np.float64).T
-        assert rel_err(out[r, :M * N].reshape(M, N), want) <= 1e-5, (shape, r)
-        assert np.all(out[r, M * N:] == 0)
+    for sc in (M * N + 5, (M * N + 3) // 4 * 4 + 8):
+        dW = capi.DeviceBuffer(R * sc * 4)
+        dW.zero()
+        capi.check(lib.mi_hgemm_tn(R, M, N, K, dAt.ptr, K, sa, dBt.ptr, K, sb, dW.ptr, N, sc, None))
+        capi.check(lib.mi_stream_sync(None))
+        out = dW.to_numpy((R, sc))
+        for r in range(R):
+            want = At[r, :M * K].reshape(M, K).astype(np.float64) @ Bt[r, :N * K].reshape(N, K).astype(np.float64).T
+            assert rel_err(out[r, :M * N].reshape(M, N), want) <= 1e-5, (shape, r, sc)
+            assert np.all(out[r, M * N:] == 0)
 
 
 @pytest.mark.parametrize("shape", [(130, 70, 100), (64, 64, 64), (33, 200, 17)])
