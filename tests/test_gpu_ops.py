@@ -93,6 +93,8 @@ GEMM_SHAPES = [
     (128, 128, 16), (128, 128, 320),
     # the short-K weight gradient with chained replicas at its own size (2048 x 2048 outputs, K = 256 per replica)
     (2048, 2048, 256),
+    # 144 tiles of 128 x 128: fewer than the CUs, still more than the 128 up to which half tiles are chosen
+    (1536, 1536, 32),
     (1, 1, 1), (5, 3, 7), (100, 130, 50), (129, 127, 33), (257, 64, 1000), (64, 1, 64), (1, 300, 17),
     # ragged but 16-byte aligned storage: the guarded MFMA kernels
     (132, 260, 100), (1000, 520, 200), (36, 4, 64), (300, 128, 36), (128, 300, 4),
