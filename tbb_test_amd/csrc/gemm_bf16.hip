@@ -706,6 +706,10 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     return !want_ct || (p.ct_rows % bm == 0 && p.ct_rows % 8 == 0 && al16(p.Ct) && batch == 1);
   };
   auto fits = [&](int bm, int bn, int bk) { return vec_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0; };
+  // variant 33: the automatic choice for a GEMM that shares the device with a bandwidth-bound launch
+  // on another stream (the per-layer update of the step)
+  const bool shares_device = variant == 33;
+  if (shares_device) variant = 0;
   if (variant == 0 && hgemm_is_skinny(p.M, p.N, p.K)) {
     // a layer of at most SKINNY_MAX outputs is matrix-vector work (forward: N, weight gradient: M,
     // input gradient: K); the caller makes the transposed copy and the bias gradient by itself
@@ -729,7 +733,11 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     //   4096 x 1024 x 1024  (64) 25.4 / 12.1 / 12.3 / 16.5    2048 x 1024 x 1024  (32) 24.2 / 10.0 / 10.2 / 15.1
     const long long t256 = (long long)(p.M / 256) * (p.N / 256) * batch;
     const long long t128 = (long long)(p.M / 128) * (p.N / 128) * batch;
-    if (fits(256, 256, 64) && t256 >= 144) variant = 27;  // falls back to 19 below if C or the mask is not 16-byte aligned
+    // The 256 x 256 kernel: four wavefronts of 128 x 128 with the hand-ordered K step (variant 32),
+    // 3-4 % faster than eight wavefronts of 128 x 64 (variant 27) when it has the device to itself.
+    // Beside an update launch that streams at HBM speed the eight-wavefront kernel loses less: with
+    // one wavefront per SIMD every tile load that the memory traffic delays is an idle MFMA pipe.
+    if (fits(256, 256, 64) && t256 >= 144) variant = shares_device ? 27 : 32;  // falls back to 19 below if C or the mask is not 16-byte aligned
     else if (fits(256, 256, 32) && t256 >= 256) variant = 13;
     else if (fits(128, 128, 64) && t128 > 256) variant = 18;
     else if (fits(128, 128, 32) && t128 >= 128) variant = 17;
@@ -752,7 +760,7 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
   // 1.63 ms, pairs 1.65 ms, all four in one workgroup 1.73 ms -- the tile stores of an entry have
   // one K step to drain before the next wait has to see them gone (the counter retires loads and
   // stores in order), the wavefronts stall there for longer than a workgroup turnover costs.
-  const bool x32 = variant >= 27 && variant <= 30;
+  const bool x32 = (variant >= 27 && variant <= 30) || variant == 32;
   if (x32 && !x32_ok()) variant = 19;
   p.chain = 1;
   if (EPI == EPH_F32 && batch > 1) {
@@ -762,7 +770,7 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
   p.vec_a = al16(p.A) && p.lda % 8 == 0 && p.batchA % 8 == 0;
   p.vec_b = al16(p.B) && p.ldb % 8 == 0 && p.batchB % 8 == 0;
   // column-sum partials come from the 256 x 256 direct-load kernels (wavefront tiles of 128 rows) only
-  if (p.colsum_part && !((variant == 13 || variant == 19 || variant == 25 || (variant >= 27 && variant <= 30)) && EPI != EPH_F32 && batch == 1 && p.M % 128 == 0)) p.colsum_part = nullptr;
+  if (p.colsum_part && !((variant == 13 || variant == 19 || variant == 25 || (variant >= 27 && variant <= 30) || variant == 32) && EPI != EPH_F32 && batch == 1 && p.M % 128 == 0)) p.colsum_part = nullptr;
   if (wrote_colsum) *wrote_colsum = p.colsum_part != nullptr;
   {  // the tile height decides whether the transposed output is possible; if not, drop it
     const int bm = (variant == 3 || variant == 17 || variant == 18) ? 128 : variant == 5 ? 64 : 256;  // (variants 13, 19, 25, 27 .. 30: 256)
@@ -782,6 +790,7 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     case 25: if (fits(256, 256, 64)) return launch_dma<256, 256, 64, 2, 4, EPI, 2, 0>(p, batch, s); break;
     case 27: case 29: case 30: return launch_x32(p, batch, EPI, true, s);
     case 28: return launch_x32(p, batch, EPI, false, s);
+    case 32: return launch_x32w4(p, batch, EPI, s);
     case 21: if (p.K > 0) return launch_h<128, 128, 32, 2, 2, EPI, 1, 3, true>(p, batch, s); break;
     case 22: if (p.K > 0) return launch_h<64, 64, 32, 2, 2, EPI, 1, 3, true>(p, batch, s); break;
     default: break;

@@ -141,6 +141,8 @@ __device__ __forceinline__ void ring_barrier() {
 // Launches the 256 x 256 x 64 kernel built on v_mfma_f32_16x16x32_bf16 (gemm_bf16_x32.hip); the
 // caller has checked the shape and alignment rules listed there.  epi: an EpilogueH value.
 hipError_t launch_x32(HGemmArgs& p, int batch, int epi, bool prio, hipStream_t s);
+// The same tile with four wavefronts of 128 x 128 and a hand-ordered K step (same rules; no chained entries).
+hipError_t launch_x32w4(HGemmArgs& p, int batch, int epi, hipStream_t s);
 
 // gemv_bf16.hip: the same product when M, N or K is at most SKINNY_MAX, as matrix-vector passes
 // (any alignment, any epilogue; no transposed second output, no column-sum partials).

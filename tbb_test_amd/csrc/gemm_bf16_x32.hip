@@ -426,6 +426,202 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_x32(HGemmArgs p) {
   store_x32<EPI>(p, acc, m0 + wm0, n0 + wn0, lane, region, bz);
 }
 
+// ---- the same tile with four wavefronts of 128 x 128, one per SIMD -------------------------------
+// A wavefront that owns 128 x 128 of the tile reads a third fewer fragment bytes from the LDS per MFMA
+// than one that owns 128 x 64, and the matrix cores of this device are power-limited: what the LDS
+// does not draw, the clock gets.  With one wavefront per SIMD, though, nothing covers a wait, so the
+// whole K step is written out as volatile asm statements, which the compiler keeps in source order:
+//   * 64 accumulator blocks (256 registers) live in AGPRs and every MFMA accumulates in place (left
+//     to itself the compiler moves them between the two register files around the MFMAs: 416 moves
+//     per K step);
+//   * a step is four sub-chunks of 32 MFMAs (K chunk 0 / 1 times the lower / upper four 16-row
+//     blocks); the fragments of the next sub-chunk are read one ds_read_b128 after every second MFMA
+//     and waited for once, at the end of the sub-chunk, so no MFMA ever waits for a read issued
+//     right in front of it;
+//   * the 16 tile loads of a wavefront and step go out one after every fifth MFMA, starting behind the
+//     barrier that frees their buffer: each direct-to-LDS load holds up the wavefront that issues it,
+//     and spread like this the MFMA already in the pipe covers most of it (all 16 in two bursts:
+//     +9 %; one per 2 / 3 / 4 / 6 MFMAs: +12 / +5 / +0.5 / +1 %);
+//   * the counters are waited for by hand (the compiler does not see these loads and reads).
+// Measured on 16384 x 8192 x 8192 against the eight-wavefront kernel above on the same box and data:
+// 1450-1512 us against 1477-1584 us (2-5 % less; boxes differ).  The same loop with its tile loads
+// taken out runs 1196-1290 us, with loads that always hit the caches 1342-1490 us.
+// Prologue / epilogue as above; the epilogue runs store_x32 once per 64-column half.
+constexpr int W4_NW = 4, W4_WN = 2;
+constexpr int W4_WTN = BN / W4_WN;                 // 128 columns per wavefront
+constexpr int W4_PB = W4_WTN / 16;                 // 8 register-side (n) blocks
+constexpr int W4_NI = BM / (RPI * W4_NW);          // 8 load instructions per wavefront, operand and tile
+constexpr int W4_SP = 5;                           // a tile load after every fifth MFMA ...
+constexpr int W4_FIRST = (4 * W4_PB - W4_SP / 2 + W4_SP - 1) / W4_SP;  // ... so many of a tile's 16 in the first sub-chunk of their window
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+
+template <int EPI>
+__global__ __launch_bounds__(W4_NW * 64) void gemm_bf16_x32w4(HGemmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) u16 smem_x[];
+  const unsigned lds_base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)((__attribute__((address_space(3))) const void*)smem_x));
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, kg = lane >> 4;
+  constexpr bool NAT = EPI == EPH_F32;  // fp32 results: natural row order of the B tile, as in the kernel above
+  const int wm0 = (wave / W4_WN) * WTM, wn0 = (wave % W4_WN) * W4_WTN;
+
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int bz = blockIdx.z;
+
+  const int lrow = lane / VPR, pc = lane % VPR;
+  unsigned offa[W4_NI], offb[W4_NI];
+#pragma unroll
+  for (int j = 0; j < W4_NI; ++j) {
+    const int row = (j * W4_NW + wave) * RPI + lrow;
+    offa[j] = 2u * ((unsigned)row * (unsigned)p.lda + (unsigned)(pc ^ swz_a(row)) * 8u);
+    offb[j] = 2u * ((unsigned)row * (unsigned)p.ldb + (unsigned)(pc ^ (NAT ? swz_a(row) : swz_b(row))) * 8u);
+  }
+  // the operand bases as scalar values (the builtin returns int: widen as unsigned)
+  auto uniform64 = [](const void* q) {
+    const unsigned long long b = reinterpret_cast<unsigned long long>(q);
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b), hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+    return ((unsigned long long)hi << 32) | lo;
+  };
+  unsigned long long sa = uniform64(p.A + (size_t)bz * p.batchA + (size_t)m0 * p.lda);
+  unsigned long long sb = uniform64(p.B + (size_t)bz * p.batchB + (size_t)n0 * p.ldb);
+  auto load_s = [](unsigned long long sbase, unsigned lane_off, unsigned lds_addr) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(lane_off), "s"(sbase) : "memory", "m0");
+  };
+  // load i of a tile's 16 (A's eight, then B's eight) into ring buffer buf; the base moves on to the
+  // next K step behind an operand's last load
+  auto tile_load = [&](auto i_c, int buf) __attribute__((always_inline)) {
+    constexpr int i = decltype(i_c)::value;
+    if constexpr (i < W4_NI) {
+      load_s(sa, offa[i], lds_base + 2u * (unsigned)(buf * A_ELEMS + (i * W4_NW + wave) * RPI * BK));
+      if (i == W4_NI - 1) sa += 2 * BK;
+    } else {
+      constexpr int j = i - W4_NI;
+      load_s(sb, offb[j], lds_base + 2u * (unsigned)(2 * A_ELEMS + buf * B_ELEMS + (j * W4_NW + wave) * RPI * BK));
+      if (j == W4_NI - 1) sb += 2 * BK;
+    }
+  };
+
+  unsigned q_addr[2], p_addr[2];
+#pragma unroll
+  for (int kc = 0; kc < 2; ++kc) {
+    const int ra = wm0 + l16, rb = NAT ? wn0 + l16 : wn0 + 8 * (l16 >> 2) + (l16 & 3);
+    q_addr[kc] = lds_base + 2u * (unsigned)(ra * BK + ((kc * 4 + kg) ^ swz_a(ra)) * 8);
+    p_addr[kc] = lds_base + 2u * (unsigned)(2 * A_ELEMS + rb * BK + ((kc * 4 + kg) ^ (NAT ? swz_a(rb) : swz_b(rb))) * 8);
+    asm volatile("" : "+v"(q_addr[kc]), "+v"(p_addr[kc]));
+  }
+  // fragment r of the 4 (m side) + 8 (n side) that sub-chunk (kc, half) multiplies, from ring buffer buf
+  i32x4_t fq[2][4], fp[2][W4_PB];
+  auto frag_read = [&](auto r_c, auto buf_c, auto kc_c, auto half_c, auto qslot_c, auto pslot_c) __attribute__((always_inline)) {
+    constexpr int r = decltype(r_c)::value, buf = decltype(buf_c)::value, kc = decltype(kc_c)::value;
+    constexpr int half = decltype(half_c)::value, qslot = decltype(qslot_c)::value, pslot = decltype(pslot_c)::value;
+    auto& fq_ = fq; auto& fp_ = fp; auto& qa_ = q_addr; auto& pa_ = p_addr;  // (named so that the lambda captures them: operands of asm statements alone do not)
+    if constexpr (r < 4) {
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(fq_[qslot][r]) : "v"(qa_[kc]), "i"(2 * (buf * A_ELEMS + (half * 4 + r) * 16 * BK)));
+    } else {
+      constexpr int ip = r - 4;
+      asm volatile("ds_read_b128 %0, %1 offset:%2"
+                   : "=&v"(fp_[pslot][ip])
+                   : "v"(pa_[kc]), "i"(2 * (buf * B_ELEMS + (NAT ? 16 * ip : 32 * (ip >> 1) + 4 * (ip & 1)) * BK)));
+    }
+  };
+
+  // acc[h][jq][ip]: rows 16 jq .. 16 jq + 15 of the wavefront's 128, n block 4 h + ip (64-column half h)
+  f32x4 acc[2][QB][4];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int jq = 0; jq < QB; ++jq)
+#pragma unroll
+      for (int ip = 0; ip < 4; ++ip)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[h][jq][ip][r] = 0.0f;
+
+  const int nk = p.K / BK;
+  // Prologue: tile 0 whole, and of tile 1 what a step requests in the first sub-chunk of a tile's
+  // window; step 0 requests the rest like every other step.
+  static_for_h<2 * W4_NI>([&](auto ic) { tile_load(ic, 0); });
+  if (nk > 1) {
+    static_for_h<W4_FIRST>([&](auto ic) { tile_load(ic, 1); });
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(W4_FIRST));
+  } else {
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+  }
+  ring_barrier();
+  using I0 = std::integral_constant<int, 0>;
+  static_for_h<4 + W4_PB>([&](auto rc) { frag_read(rc, I0{}, I0{}, I0{}, I0{}, I0{}); });
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+
+  // Step t multiplies buffer t % 2.  Sub-chunk s uses the m-side fragments in slot s % 2 and the n-side
+  // fragments in slot s / 2 and reads those of sub-chunk s + 1 (s = 3: of step t + 1, from the other
+  // buffer) into the other slots.  Behind sub-chunk 2: every read of this buffer and tile t+1 are
+  // waited for, then the barrier; the window of tile t+2 (into this buffer) opens with sub-chunk 3 and
+  // runs on through sub-chunks 0 and 1 of step t+1.
+  auto step = [&](int t, auto cur_c, auto steady_c) __attribute__((always_inline)) {
+    constexpr int cur = decltype(cur_c)::value;
+    constexpr bool steady = decltype(steady_c)::value;  // tiles t+1 and t+2 exist
+    static_for_h<4>([&](auto s_c) {
+      constexpr int s = decltype(s_c)::value, ns = (s + 1) & 3;
+      using RBuf = std::integral_constant<int, (s == 3 ? (cur ^ 1) : cur)>;
+      using NKc = std::integral_constant<int, (ns >> 1)>;
+      using NHalf = std::integral_constant<int, (ns & 1)>;
+      using QSlot = std::integral_constant<int, (ns & 1)>;
+      using PSlot = std::integral_constant<int, ((ns >> 1) & 1)>;
+      constexpr int nreads = 4 + ((ns & 1) == 0 ? W4_PB : 0);  // the n-side fragments change with the K chunk only
+      static_for_h<4 * W4_PB>([&](auto ic) {
+        constexpr int idx = decltype(ic)::value, jj = idx / W4_PB, ip = idx % W4_PB;
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                     : "+a"(acc[ip >> 2][(s & 1) * 4 + jj][ip & 3])
+                     : "v"(fp[(s >> 1) & 1][ip]), "v"(fq[s & 1][jj]));
+        if constexpr ((idx & 1) == 1 && idx / 2 < nreads)
+          frag_read(std::integral_constant<int, idx / 2>{}, RBuf{}, NKc{}, NHalf{}, QSlot{}, PSlot{});
+        constexpr int w = ((s + 1) & 3) * 4 * W4_PB + idx;  // position in the window that sub-chunk 3 opens
+        if constexpr (s != 2 && w % W4_SP == W4_SP / 2 && w / W4_SP < 2 * W4_NI) {
+          // s == 3: tile t+2 into this buffer; s == 0, 1: the rest of tile t+1 into the other one
+          if (s == 3 ? (steady || t + 2 < nk) : (steady || t + 1 < nk))
+            tile_load(std::integral_constant<int, w / W4_SP>{}, s == 3 ? cur : cur ^ 1);
+        }
+      });
+      if constexpr (s == 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    });
+  };
+  using C0 = std::integral_constant<int, 0>;
+  using C1 = std::integral_constant<int, 1>;
+  int t = 0;
+  for (; t + 4 <= nk; t += 2) {
+    step(t, C0{}, std::true_type{});
+    step(t + 1, C1{}, std::true_type{});
+  }
+  static_for_h<3>([&](auto sc) {
+    constexpr int s = decltype(sc)::value;
+    if (t + s < nk) step(t + s, std::integral_constant<int, s % 2>{}, std::false_type{});
+  });
+  // the compiler does not know that MFMAs have just written the accumulators it is about to read
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+  unsigned char* region = nullptr;
+  if (EPI != EPH_F32 && p.Ct) {
+    __syncthreads();  // every wavefront is done with the operand tiles: the LDS is free for the staging
+    region = reinterpret_cast<unsigned char*>(smem_x) + (size_t)wave * STAGE_REGION;
+  }
+  store_x32<EPI>(p, acc[0], m0 + wm0, n0 + wn0, lane, region, bz);
+  store_x32<EPI>(p, acc[1], m0 + wm0, n0 + wn0 + 64, lane, region, bz);
+}
+
+template <int EPI>
+hipError_t launch_w4(HGemmArgs& p, int batch, hipStream_t s) {
+  p.tiles_m = p.M / BM;
+  p.tiles_n = p.N / BN;
+  p.chain = 1;
+  auto kern = gemm_bf16_x32w4<EPI>;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), LDS_BYTES); e != hipSuccess) return e;
+  launch_kernel(kern, dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(W4_NW * 64), LDS_BYTES, s, p);
+  return hipGetLastError();
+}
+
 template <int EPI, int PRIO>
 hipError_t launch_one(HGemmArgs& p, int batch, hipStream_t s) {
   p.tiles_m = p.M / BM;
@@ -463,6 +659,15 @@ hipError_t launch_prio(HGemmArgs& p, int batch, int epi, hipStream_t s) {
 
 hipError_t launch_x32(HGemmArgs& p, int batch, int epi, bool prio, hipStream_t s) {
   return prio ? launch_prio<1>(p, batch, epi, s) : launch_prio<0>(p, batch, epi, s);
+}
+
+hipError_t launch_x32w4(HGemmArgs& p, int batch, int epi, hipStream_t s) {
+  switch (epi) {
+    case EPH_F32: return launch_w4<EPH_F32>(p, batch, s);
+    case EPH_BIAS_RELU: return launch_w4<EPH_BIAS_RELU>(p, batch, s);
+    case EPH_MASK: return launch_w4<EPH_MASK>(p, batch, s);
+    default: return launch_w4<EPH_BF16>(p, batch, s);
+  }
 }
 
 }  // namespace mi

@@ -61,9 +61,10 @@ HSHAPES = [(64, 64, 32), (128, 128, 64), (256, 256, 96), (512, 256, 128), (256, 
            # 288 tiles of 128 x 128 (72 of 256 x 256): what the automatic choice gives to the eight-wavefront
            # 128 x 128 x 64 instance; 144 tiles of 256 x 256: the smallest problem it gives to the 256 x 256 kernel
            (2048, 2304, 128), (3072, 3072, 64)]
-HVARIANTS = [0, 3, 4, 5, 13, 17, 18, 19, 21, 22, 25, 27, 28, 29, 30]
+HVARIANTS = [0, 3, 4, 5, 13, 17, 18, 19, 21, 22, 25, 27, 28, 29, 30, 32]
 # 21, 22: guarded any-shape MFMA instances; 25: 19 without wave priorities; 27, 28: 16x16x32 MFMAs;
-# 29 / 30: 27 with all / pairs of the batch entries of a weight gradient chained in one workgroup
+# 29 / 30: 27 with all / pairs of the batch entries of a weight gradient chained in one workgroup;
+# 32: the 256 x 256 x 64 tile with four wavefronts of 128 x 128 and a hand-ordered K step
 
 
 @pytest.mark.parametrize("variant", HVARIANTS)
@@ -418,7 +419,7 @@ def test_bf16_step_matches_fp32_oracle(name, flags):
     _check_bf16_step(nf, B, R, flags)
 
 
-@pytest.mark.parametrize("variant", [13, 17, 18, 19, 25, 27, 28])
+@pytest.mark.parametrize("variant", [13, 17, 18, 19, 25, 27, 28, 32])
 @pytest.mark.parametrize("flags", [capi.FLAG_NO_GRAPH, 0])
 def test_bf16_step_on_the_large_tile_kernels(variant, flags):
     """The direct-load kernels (256 x 256 and 128 x 128 tiles), which small models never pick by
