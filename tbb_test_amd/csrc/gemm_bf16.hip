@@ -735,8 +735,12 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     const long long t128 = (long long)(p.M / 128) * (p.N / 128) * batch;
     // The 256 x 256 kernel: four wavefronts of 128 x 128 with the hand-ordered K step (variant 32),
     // 3-4 % faster than eight wavefronts of 128 x 64 (variant 27) when it has the device to itself.
-    // Beside an update launch that streams at HBM speed the eight-wavefront kernel loses less: with
-    // one wavefront per SIMD every tile load that the memory traffic delays is an idle MFMA pipe.
+    // Beside an update launch the eight-wavefront kernel is the better one: its two wavefronts per SIMD
+    // take 2 x 206-211 of the 512 registers, which leaves room for a wavefront of the update kernel
+    // that is launched for this case (76 registers, 16 KB of LDS) on the same CU, while the
+    // bf16-result instances of the four-wavefront kernel take the whole register file and the update's
+    // workgroups have to take whole CUs in turns with the GEMM's.  (Its fp32-result instance needs
+    // 372 registers and shares a CU with the update like the eight-wavefront kernel does.)
     if (fits(256, 256, 64) && t256 >= 144) variant = shares_device ? 27 : 32;  // falls back to 19 below if C or the mask is not 16-byte aligned
     else if (fits(256, 256, 32) && t256 >= 256) variant = 13;
     else if (fits(128, 128, 64) && t128 > 256) variant = 18;

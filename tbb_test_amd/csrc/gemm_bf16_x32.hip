@@ -26,6 +26,10 @@
 //
 // The transposed per-replica copy (Ct) wants runs along m instead: it goes through the then idle
 // LDS, one private region per wavefront, as in gemm_bf16_dma.
+//
+// Two kernels share this tile, layout and epilogue: gemm_bf16_x32 (eight wavefronts of 128 x 64, the
+// K step ordered by the compiler; also the chained-replica instance) and gemm_bf16_x32w4 (four
+// wavefronts of 128 x 128, the K step written out instruction by instruction), further down.
 #include <hip/hip_runtime.h>
 
 #include "gemm_bf16_common.h"
