@@ -352,7 +352,7 @@ def measure_config(config, args, steps, warmup, info, np, capi, hostlib, min_loo
         "reduce_gbps": round(upd_gbps, 1),
         "weights_finite": finite,
         "roofline": {"kernel": "gemm_f32_dma (nt, nn, tn)" if dtype == "f32" else
-                               "gemm_bf16_x32w4, gemm_bf16_x32 for an input gradient beside an update launch (spans of the weight gradient include the column-sum fold or row-sum "
+                               "gemm_bf16_x32w4 (spans of the weight gradient include the column-sum fold or row-sum "
                                "kernel of the bias gradient and, for operands no GEMM epilogue wrote transposed, the "
                                "transpose launches)",
                      "bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": peak, "unit": "TFLOP/s",

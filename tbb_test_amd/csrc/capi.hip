@@ -140,8 +140,6 @@ struct mi_mlp {
   bool neg_lr_valid = false;
   // what the last enqueue_step decided (mi_mlp_get_schedule)
   bool last_dual = false, last_per_layer = false, last_paired = false;
-  // set by enqueue_step around the GEMMs that run while an update launch of another layer is in flight on the other stream
-  bool beside_update = false;
 
   size_t esize() const { return dtype == MI_BF16 ? 2 : 4; }
   size_t maxw() const {
@@ -329,8 +327,7 @@ int op_dgrad(mi_mlp* h, int l, hipStream_t s) {
     float* cp = (l > 0 && h->B % 128 == 0) ? h->colpart[(l - 1) % h->ndz] : nullptr;  // and its column sums
     e = mi::hgemm_nt(1, h->MB, h->nf[l], h->nf[l + 1], (const uint16_t*)dz_of_layer(h, l), h->nf[l + 1], 0,
                      h->params16T + h->woff[l], h->nf[l + 1], 0, out, h->nf[l], 0, mask ? 2 : 3, nullptr, 0,
-                     (const uint16_t*)mask, h->nf[l], s, (g_hvariant == 0 && h->beside_update) ? 33 : (int)g_hvariant, ct, h->B,
-                     &wrote, cp, &wrote_cs);
+                     (const uint16_t*)mask, h->nf[l], s, g_hvariant, ct, h->B, &wrote, cp, &wrote_cs);
     if (l > 0) {
       h->dzT_fused[(l - 1) % h->ndz] = wrote;
       h->dzT_fused_layer[l - 1] = wrote;
@@ -577,15 +574,13 @@ int enqueue_step(mi_mlp* h, float lr) {
   // update launch: durations of kernels that overlap cannot be attributed to a kernel.
   // (per-kernel timing keeps the separate launches so that every phase has its own figures)
   const bool paired = small_model(h) && !h->timing;
-  const bool per_layer_sched = (h->flags & MI_FLAG_PER_LAYER_UPDATE) != 0 && !small_model(h);  // what the untimed step does
-  const bool per_layer = per_layer_sched && !h->timing;
+  const bool per_layer = (h->flags & MI_FLAG_PER_LAYER_UPDATE) != 0 && !h->timing && !paired;
   // Two backward streams pay while a GEMM launch leaves CUs idle at its start and end, i.e. up to
   // a few tiles per CU (configs 2 and 4: 256 tiles of 128 x 128 per input-gradient launch, 3-5 %
   // faster with two streams).  GEMMs with many tiles per CU only get in each other's way (config
   // 3, 1024 tiles: 11.32 ms with one backward stream, 11.47 ms with two; config 5: 45.9 / 47.1 ms).
   const bool crowded = (long long)(h->MB / 128) * (long long)(h->maxw() / 128) >= 1024;
-  const bool dual_sched = !(h->flags & MI_FLAG_SERIAL_BACKWARD) && !crowded && !small_model(h);
-  const bool dual = dual_sched && !h->timing;
+  const bool dual = !(h->flags & MI_FLAG_SERIAL_BACKWARD) && !h->timing && !crowded && !paired;
   if (!h->timing) {  // the per-kernel timing pass is not the schedule mi_mlp_get_schedule reports
     h->last_dual = dual;
     h->last_per_layer = per_layer;
@@ -616,14 +611,7 @@ int enqueue_step(mi_mlp* h, float lr) {
         if (l + 2 <= h->L - 1) MI_HIP(hipStreamWaitEvent(s, h->ev_wgrad[l + 2], 0));
       }
     }
-    // bf16 on one backward stream: in the untimed step the update of layer l+1 has just been put on
-    // the other stream and runs beside this input-gradient GEMM (the weight gradient behind it is
-    // better off on the four-wavefront kernel either way: config 5 38.24 against 38.50 ms).  The
-    // per-kernel timing pass takes the same choice, so that it times the kernels the step runs.
-    h->beside_update = per_layer_sched && !dual_sched && l < h->L - 1;
-    rc = op_dgrad(h, l, s);
-    h->beside_update = false;
-    if (rc) return rc;
+    if ((rc = op_dgrad(h, l, s))) return rc;
     if (dgrad_first)
       if ((rc = op_wgrad(h, l, s, true))) return rc;
     if (dual || per_layer) {

@@ -706,10 +706,6 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     return !want_ct || (p.ct_rows % bm == 0 && p.ct_rows % 8 == 0 && al16(p.Ct) && batch == 1);
   };
   auto fits = [&](int bm, int bn, int bk) { return vec_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0; };
-  // variant 33: the automatic choice for a GEMM that shares the device with a bandwidth-bound launch
-  // on another stream (the per-layer update of the step)
-  const bool shares_device = variant == 33;
-  if (shares_device) variant = 0;
   if (variant == 0 && hgemm_is_skinny(p.M, p.N, p.K)) {
     // a layer of at most SKINNY_MAX outputs is matrix-vector work (forward: N, weight gradient: M,
     // input gradient: K); the caller makes the transposed copy and the bias gradient by itself
@@ -734,14 +730,12 @@ static hipError_t dispatch_h(HGemmArgs& p, int batch, hipStream_t s, int variant
     const long long t256 = (long long)(p.M / 256) * (p.N / 256) * batch;
     const long long t128 = (long long)(p.M / 128) * (p.N / 128) * batch;
     // The 256 x 256 kernel: four wavefronts of 128 x 128 with the hand-ordered K step (variant 32),
-    // 3-4 % faster than eight wavefronts of 128 x 64 (variant 27) when it has the device to itself.
-    // Beside an update launch the eight-wavefront kernel is the better one: its two wavefronts per SIMD
-    // take 2 x 206-211 of the 512 registers, which leaves room for a wavefront of the update kernel
-    // that is launched for this case (76 registers, 16 KB of LDS) on the same CU, while the
-    // bf16-result instances of the four-wavefront kernel take the whole register file and the update's
-    // workgroups have to take whole CUs in turns with the GEMM's.  (Its fp32-result instance needs
-    // 372 registers and shares a CU with the update like the eight-wavefront kernel does.)
-    if (fits(256, 256, 64) && t256 >= 144) variant = shares_device ? 27 : 32;  // falls back to 19 below if C or the mask is not 16-byte aligned
+    // 3-4 % faster than eight wavefronts of 128 x 64 (variant 27).  Both leave registers free for a
+    // wavefront of the update kernel that the step launches beside a GEMM (76 registers, 16 KB of LDS:
+    // the eight-wavefront kernel takes 2 x 206-211 of a SIMD's 512, this one 372-396 since its
+    // epilogue reads the accumulators out of the AGPRs row block by row block), so the two share CUs
+    // instead of taking them in turns.
+    if (fits(256, 256, 64) && t256 >= 144) variant = 32;  // falls back to 19 below if C or the mask is not 16-byte aligned
     else if (fits(256, 256, 32) && t256 >= 256) variant = 13;
     else if (fits(128, 128, 64) && t128 > 256) variant = 18;
     else if (fits(128, 128, 32) && t128 >= 128) variant = 17;

@@ -61,7 +61,7 @@ __device__ __forceinline__ int swz_b(int row) { return ((row >> 3) & 3) * 2 + ((
 
 // Epilogue of one wavefront: acc[jq][ip] is the 16 x 16 block of rows row0 + 16 jq + lane % 16 and
 // the four columns described at the top of the file.
-template <int EPI>
+template <int EPI, bool ACC_IN_AGPRS = false>
 __device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][PB], int row0, int colw, int lane,
                                           unsigned char* region, int bz) {
   const int l16 = lane & 15, q = lane >> 4;
@@ -111,8 +111,15 @@ __device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][P
         const int col = colw + 32 * h + 8 * q;
         const float(&bias_v)[8] = bias_all[h];
         float v[8];
+        if constexpr (ACC_IN_AGPRS) {
+          // read out here and nowhere earlier: left to the compiler, all 256 accumulators are copied to
+          // VGPRs in front of the epilogue, which then needs the whole register file
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = acc[jq][2 * h + (e >> 2)][e & 3];
+          for (int e = 0; e < 8; ++e) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[jq][2 * h + (e >> 2)][e & 3]));
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = acc[jq][2 * h + (e >> 2)][e & 3];
+        }
         if (EPI == EPH_BIAS_RELU) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
@@ -135,6 +142,7 @@ __device__ __forceinline__ void store_x32(const HGemmArgs& p, f32x4 (&acc)[QB][P
         }
         pk[jq][h] = out;
         *reinterpret_cast<u32x4*>(ch + (size_t)row * p.ldc + col) = out;
+        if constexpr (ACC_IN_AGPRS) asm volatile("" : : "v"(out));  // (volatile statements keep their order: this row's work stays in front of the next row's reads)
       }
     }
     if (p.colsum_part) {
@@ -610,8 +618,12 @@ __global__ __launch_bounds__(W4_NW * 64) void gemm_bf16_x32w4(HGemmArgs p) {
     __syncthreads();  // every wavefront is done with the operand tiles: the LDS is free for the staging
     region = reinterpret_cast<unsigned char*>(smem_x) + (size_t)wave * STAGE_REGION;
   }
-  store_x32<EPI>(p, acc[0], m0 + wm0, n0 + wn0, lane, region, bz);
-  store_x32<EPI>(p, acc[1], m0 + wm0, n0 + wn0 + 64, lane, region, bz);
+  // what the epilogue derives its addresses from is made opaque here, so that none of it is computed
+  // ahead of the K loop and kept in registers through it
+  int lane_e = lane, row_e = m0 + wm0, col_e = n0 + wn0;
+  asm volatile("" : "+v"(lane_e), "+s"(row_e), "+s"(col_e));
+  store_x32<EPI, EPI != EPH_F32>(p, acc[0], row_e, col_e, lane_e, region, bz);
+  store_x32<EPI, EPI != EPH_F32>(p, acc[1], row_e, col_e + 64, lane_e, region, bz);
 }
 
 template <int EPI>

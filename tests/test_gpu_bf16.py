@@ -61,11 +61,10 @@ HSHAPES = [(64, 64, 32), (128, 128, 64), (256, 256, 96), (512, 256, 128), (256, 
            # 288 tiles of 128 x 128 (72 of 256 x 256): what the automatic choice gives to the eight-wavefront
            # 128 x 128 x 64 instance; 144 tiles of 256 x 256: the smallest problem it gives to the 256 x 256 kernel
            (2048, 2304, 128), (3072, 3072, 64)]
-HVARIANTS = [0, 3, 4, 5, 13, 17, 18, 19, 21, 22, 25, 27, 28, 29, 30, 32, 33]
+HVARIANTS = [0, 3, 4, 5, 13, 17, 18, 19, 21, 22, 25, 27, 28, 29, 30, 32]
 # 21, 22: guarded any-shape MFMA instances; 25: 19 without wave priorities; 27, 28: 16x16x32 MFMAs;
 # 29 / 30: 27 with all / pairs of the batch entries of a weight gradient chained in one workgroup;
-# 32: the 256 x 256 x 64 tile with four wavefronts of 128 x 128 and a hand-ordered K step;
-# 33: the automatic choice for a GEMM that runs beside an update launch (what the step asks for there)
+# 32: the 256 x 256 x 64 tile with four wavefronts of 128 x 128 and a hand-ordered K step
 
 
 @pytest.mark.parametrize("variant", HVARIANTS)
